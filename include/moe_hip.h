@@ -190,6 +190,9 @@ MOE_API int moe_k_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, const
  *           down-projection weight gradient
  *   dscale [R] fp32 or NULL: dscale[idx(p)] = <dy[p], act(h[p])>, the gradient of
  *           the routing weight
+ * MOE_ACT_NONE is the identity (act' = 1): experts without an activation
+ * (MLPParams.activation = None, params.py:11-15) still need the row scaling,
+ * row_scale * h and dscale.
  */
 MOE_API int moe_act_bwd(const void* h, int64_t ldh, const void* dy, int64_t lddy, void* dh,
                 int64_t lddh, const void* row_scale, const void* indices, int idx_bytes,

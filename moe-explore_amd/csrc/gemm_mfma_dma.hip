@@ -31,8 +31,8 @@
 
 #include <stdlib.h>
 
-#include <atomic>
 #include <mutex>
+#include <unordered_map>
 
 namespace moe {
 namespace {
@@ -437,8 +437,12 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
 // queue share the weight tiles they stream, and an XCD has its own L2), then from the other
 // queues, so every id is drawn whatever XCDs the launch lands on.  Word 8 of a queue set counts
 // the workgroups that are done; the last one clears the set for the next launch that uses it.
-// Launches take the sets in turn: two launches share a set only if 1024 others were issued
-// between them while the first was still running.
+// A queue set belongs to ONE stream of one device: launches on a stream run one after the
+// other, so they can share a set, and launches on different streams never do.  A launch that is
+// being captured into a graph takes no set at all (queue == nullptr: workgroup b takes the ids
+// b, b + gridDim.x, ... in order): a graph may be replayed on any stream, several times at once
+// and next to eager launches, so nothing it runs may own device state.  The same holds for a
+// process that uses more than kQueueSets streams on one device.
 constexpr int kQueueSets = 1024;
 constexpr int kQueueWords = 16;
 static_assert((kNumXcd & (kNumXcd - 1)) == 0 && kNumXcd < kQueueWords, "queue per XCD, then the counter");
@@ -460,6 +464,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void m_grouped_dma_kernel(DmaKernel
   const int home = __builtin_amdgcn_s_getreg((31 << 11) | 20) & (kNumXcd - 1);
   int tried = 0;  // queues found empty so far, the home queue first
   NextDraw next{nullptr, 0u, false};
+  int64_t static_id = blockIdx.x;  // launches without a queue set: ids in strides of the grid
   for (;;) {
     // The arguments are read from the kernel argument segment again for every tile: held in
     // scalar registers across the tiles they crowd out what the K loop keeps there.
@@ -467,7 +472,10 @@ __global__ __launch_bounds__(64 * WVM * WVN) void m_grouped_dma_kernel(DmaKernel
     asm volatile("" : "+s"(kp));
     const DmaKernelArgs* const args = (const DmaKernelArgs*)kp;
     __syncthreads();  // every wavefront is done with the LDS of the tile before
-    if (threadIdx.x == 0) {
+    if (threadIdx.x == 0 && args->queue == nullptr) {
+      *sh_next = static_id < args->s.wgs ? static_cast<int>(static_id) : -1;
+      static_id += gridDim.x;
+    } else if (threadIdx.x == 0) {
       unsigned* const queue = args->queue;
       const int total = static_cast<int>(args->s.wgs);
       int id = -1;
@@ -492,7 +500,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void m_grouped_dma_kernel(DmaKernel
     m_grouped_dma_tile<T, BM, WVM, WVN, WL, ACT>(args->g, args->s, id, next);
   }
   // (every workgroup ends here: each queue runs dry after s.wgs / 8 draws)
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0 && ka.queue != nullptr) {
     unsigned* const queue = ka.queue;
     __threadfence();
     if (atomicAdd(&queue[kNumXcd], 1u) == gridDim.x - 1) {
@@ -501,46 +509,50 @@ __global__ __launch_bounds__(64 * WVM * WVN) void m_grouped_dma_kernel(DmaKernel
   }
 }
 
-// The queue set of the next launch on the current device (nullptr after fail()) and the
-// number of compute units of that device.  Every device holds its own copy of g_tile_queues.
-unsigned* next_queue_set(int* cus) {
+// The queue set of `stream` on the current device and the number of compute units of that
+// device.  *queue stays nullptr (ids in strides of the grid, no device state) while the stream
+// is being captured and when the device has handed out all its sets.  Every device holds its
+// own copy of g_tile_queues.  Returns MOE_OK or the status of fail().
+int queue_set_of(hipStream_t stream, unsigned** queue, int* cus) {
   struct DeviceQueues {
     unsigned* base = nullptr;
     int cus = 0;
+    std::unordered_map<hipStream_t, unsigned> set_of_stream;
   };
   constexpr int kMaxDevices = 64;
   static DeviceQueues per_device[kMaxDevices];
   static std::mutex lock;
-  static std::atomic<unsigned> next_set{0};
+  *queue = nullptr;
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
-  if (err != hipSuccess || dev < 0 || dev >= kMaxDevices) {
-    fail(MOE_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(err));
-    return nullptr;
-  }
-  DeviceQueues dq;
-  {
-    std::lock_guard<std::mutex> hold(lock);
-    if (per_device[dev].base == nullptr) {
-      void* p = nullptr;
-      err = hipGetSymbolAddress(&p, HIP_SYMBOL(g_tile_queues));
-      if (err != hipSuccess || p == nullptr) {
-        fail(MOE_ERR_HIP, "hipGetSymbolAddress(tile queues): %s", hipGetErrorString(err));
-        return nullptr;
-      }
-      int n = 0;
-      err = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
-      if (err != hipSuccess || n < 1) {
-        fail(MOE_ERR_HIP, "hipDeviceGetAttribute(compute units): %s", hipGetErrorString(err));
-        return nullptr;
-      }
-      per_device[dev].cus = n;
-      per_device[dev].base = static_cast<unsigned*>(p);
-    }
-    dq = per_device[dev];
+  if (err != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(MOE_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(err));
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  err = hipStreamIsCapturing(stream, &capture);
+  if (err != hipSuccess) return fail(MOE_ERR_HIP, "hipStreamIsCapturing: %s", hipGetErrorString(err));
+  std::lock_guard<std::mutex> hold(lock);
+  DeviceQueues& dq = per_device[dev];
+  if (dq.base == nullptr) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(g_tile_queues));
+    if (err != hipSuccess || p == nullptr)
+      return fail(MOE_ERR_HIP, "hipGetSymbolAddress(tile queues): %s", hipGetErrorString(err));
+    int n = 0;
+    err = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+    if (err != hipSuccess || n < 1)
+      return fail(MOE_ERR_HIP, "hipDeviceGetAttribute(compute units): %s", hipGetErrorString(err));
+    dq.cus = n;
+    dq.base = static_cast<unsigned*>(p);
   }
   *cus = dq.cus;
-  return dq.base + static_cast<size_t>(next_set.fetch_add(1) % kQueueSets) * kQueueWords;
+  if (capture != hipStreamCaptureStatusNone) return MOE_OK;
+  auto it = dq.set_of_stream.find(stream);
+  if (it == dq.set_of_stream.end()) {
+    if (dq.set_of_stream.size() >= static_cast<size_t>(kQueueSets)) return MOE_OK;
+    it = dq.set_of_stream.emplace(stream, static_cast<unsigned>(dq.set_of_stream.size())).first;
+  }
+  *queue = dq.base + static_cast<size_t>(it->second) * kQueueWords;
+  return MOE_OK;
 }
 
 // Sets the kernel's dynamic LDS limit on first use and launches it with one workgroup per
@@ -559,13 +571,17 @@ int launch_kernel(const MGemmArgs& g, const Sched& s, dim3 grid, int threads, si
     configured = true;
   }
   int cus = 0;
-  unsigned* const queue = next_queue_set(&cus);
-  if (queue == nullptr) return MOE_ERR_HIP;
+  unsigned* queue = nullptr;
+  const int rc = queue_set_of(stream, &queue, &cus);
+  if (rc != MOE_OK) return rc;
   DmaKernelArgs ka;
   ka.g = g;
   ka.s = s;
   ka.queue = queue;
-  const unsigned wgs = grid.x < static_cast<unsigned>(cus) ? grid.x : static_cast<unsigned>(cus);
+  // (a multiple of the XCD count, so that ids taken in strides of the grid stay on their XCD)
+  unsigned wgs = static_cast<unsigned>(cus) / kNumXcd * kNumXcd;
+  if (wgs == 0) wgs = static_cast<unsigned>(cus);
+  if (grid.x < wgs) wgs = grid.x;
   Kernel<<<dim3(wgs), threads, lds, stream>>>(ka);
   return MOE_OK;
 }

@@ -358,7 +358,6 @@ extern "C" int moe_act_bwd(const void* h, int64_t ldh, const void* dy, int64_t l
                            int64_t N, int act, int dtype, moe_stream_t stream_) {
   clear_error();
   MOE_REQUIRE(R >= 0 && N >= 0, "negative size");
-  MOE_REQUIRE(act != MOE_ACT_NONE, "activation gradient of the identity is not an op");
   MOE_REQUIRE(indices == nullptr || idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8");
   if (R == 0 || N == 0) return MOE_OK;
   MOE_REQUIRE(h && dy && dh, "null pointer");

@@ -10,9 +10,12 @@ gradient; the reference itself is forward-only.
 ``topk_moe_torch`` is the plain-PyTorch per-expert loop that the reference ships
 as its comparison implementation (``:67-102``); it is not used by the HIP path.
 """
+import weakref
+
 import torch
 
 from moe_explore.params import MOEParams, MLPParams, GLUParams, GLUInterleavedParams
+from moe_explore.tracing import scope
 from moe_explore.functional.activation import activation, activation_name, is_glu
 from moe_explore.functional.scale_and_reduce import scale_and_reduce
 from moe_explore.router import router
@@ -31,17 +34,74 @@ def interleave_glu_weights(gate_weight, up_weight):
     """[E, d, ff] gate and up -> [E, d, 2*ff] with gate in the even and up in the odd
     columns, the layout the GLU epilogue reads (``functional/activation.py:19-20``)."""
     e, d, ff = gate_weight.shape
-    return torch.stack((gate_weight, up_weight), dim=-1).reshape(e, d, 2 * ff)
+    out = torch.empty((e, d, 2 * ff), device=gate_weight.device, dtype=gate_weight.dtype)
+    out[:, :, 0::2] = gate_weight
+    out[:, :, 1::2] = up_weight
+    return out
+
+
+def to_interleaved(ep):
+    """Load-time conversion of separate gate / up weights (``params.py:16-21``, the layout of
+    Hugging Face checkpoints) into the record the kernels read directly.  Training code
+    should convert once and keep the result as its parameter: the weight gradient then
+    comes back in the same interleaved layout and nothing is copied per step."""
+    if isinstance(ep, GLUParams):
+        return GLUInterleavedParams(interleave_glu_weights(ep.gate_weight, ep.up_weight),
+                                    ep.down_weight, ep.activation)
+    return ep
+
+
+# interleaved copies of GLUParams weights, one per (gate, up) pair, rebuilt only when one of
+# the two tensors has been written since (their version counters)
+_interleaved_cache = {}
+_INTERLEAVED_CACHE_MAX = 256
+
+
+def _cached_interleave(gate, up):
+    key = (id(gate), id(up))
+    hit = _interleaved_cache.get(key)
+    if hit is not None:
+        g_ref, u_ref, g_ver, u_ver, ptrs, w = hit
+        if g_ref() is gate and u_ref() is up and g_ver == gate._version and \
+                u_ver == up._version and ptrs == (gate.data_ptr(), up.data_ptr()):
+            return w
+    w = interleave_glu_weights(gate.detach(), up.detach())
+    if len(_interleaved_cache) >= _INTERLEAVED_CACHE_MAX:
+        _interleaved_cache.clear()
+    drop = lambda _, key=key: _interleaved_cache.pop(key, None)
+    _interleaved_cache[key] = (weakref.ref(gate, drop), weakref.ref(up, drop), gate._version,
+                               up._version, (gate.data_ptr(), up.data_ptr()), w)
+    return w
+
+
+class _InterleaveFunction(torch.autograd.Function):
+    """Differentiable view of the cached interleaved copy: the gradient of weight1 goes
+    back to gate and up as its even and odd columns."""
+
+    @staticmethod
+    def forward(ctx, gate, up):
+        return _cached_interleave(gate, up).detach()
+
+    @staticmethod
+    def backward(ctx, dw):
+        return dw[:, :, 0::2], dw[:, :, 1::2]
 
 
 def expert_weights(ep):
-    """(weight1, weight2, activation) of any of the reference's FFN parameter records."""
+    """(weight1, weight2, activation) of any of the reference's FFN parameter records.
+    Separate gate / up weights are interleaved once and the copy is reused until either
+    tensor is written again."""
     if isinstance(ep, MLPParams):
         return ep.weight1, ep.weight2, ep.activation
     if isinstance(ep, GLUInterleavedParams):
         return ep.interleaved_weight, ep.down_weight, ep.activation
     if isinstance(ep, GLUParams):
-        return interleave_glu_weights(ep.gate_weight, ep.up_weight), ep.down_weight, ep.activation
+        gate, up = ep.gate_weight, ep.up_weight
+        if torch.is_grad_enabled() and (gate.requires_grad or up.requires_grad):
+            w1 = _InterleaveFunction.apply(gate, up)
+        else:
+            w1 = _cached_interleave(gate, up)
+        return w1, ep.down_weight, ep.activation
     raise ValueError(f"Unsupported expert parameter type: {type(ep)}")
 
 
@@ -64,18 +124,22 @@ class _ExpertsFunction(torch.autograd.Function):
         T = x.size(0)
         need_grad = any(ctx.needs_input_grad[:4])
         p1 = MGroupedGEMMParams(w1, group_indices, indices, True, False, T, topk, activation=act)
-        if need_grad:
-            a, h = m_grouped_gemm(x, p1, save_preact=True)
-        else:
-            a, h = m_grouped_gemm(x, p1), None
+        with scope("fused_grouped_glu"):
+            if need_grad and act is not None:
+                a, h = m_grouped_gemm(x, p1, save_preact=True)
+            else:
+                a = m_grouped_gemm(x, p1)
+                h = a if need_grad else None  # identity activation: A is its own pre-activation
         # down projection stored in slot order, then the top-k weighted sum
         # (reference topk_moe.py:36-54); the fp32-atomic fused combine of
         # m_grouped_gemm(combine=True) is slower than this second pass on MI355X
         p2 = MGroupedGEMMParams(w2, group_indices, indices, False, True, T, topk, scales=scores)
         ks = _ksplit_for(T * topk, w2.size(0), w2.size(2), w2.size(1))
-        y = m_grouped_gemm(a, p2, ksplit=ks)
+        with scope("down_grouped_gemm"):
+            y = m_grouped_gemm(a, p2, ksplit=ks)
         ks = y.size(0) // (T * topk)
-        out = scale_and_reduce(y, scores, T, topk, y.size(1), nsplit=ks)
+        with scope("scale_and_reduce"):
+            out = scale_and_reduce(y, scores, T, topk, y.size(1), nsplit=ks)
         if need_grad:
             ctx.save_for_backward(x, w1, w2, scores, group_indices, indices, h)
             ctx.act, ctx.topk = act, topk
@@ -88,9 +152,6 @@ class _ExpertsFunction(torch.autograd.Function):
         dout = dout.contiguous()
         # G[p] = dout[token(p)] @ w2[e]^T
         need_dscore = ctx.needs_input_grad[3]
-        if act is None:
-            # identity activation: dH = score * G, A = H
-            raise NotImplementedError("experts without an activation have no backward here")
         fused = None
         if is_glu(act):
             # G is turned into dH, s*A and dscore in the GEMM's epilogue and never stored
@@ -102,6 +163,7 @@ class _ExpertsFunction(torch.autograd.Function):
         else:
             pg = MGroupedGEMMParams(w2, gi, idx, True, False, T, topk)
             g = m_grouped_gemm(dout, pg, transpose_weight=True)
+            # (identity activation: dH = s * G, s * A = s * H, dscore = <G, H>)
             dh, a_scaled, dscale = act_bwd(h, g, act, row_scale=scores, permute_indices=idx,
                                            want_y_scaled=True, want_dscale=need_dscore)
         dw1 = dw2 = dx = dscores = None
@@ -127,22 +189,38 @@ class _ExpertsFunction(torch.autograd.Function):
 def routed_experts(x, weight1, weight2, topk_scores, topk_indices, num_experts, topk, act):
     """Experts + combine for given routing decisions (differentiable in ``x``, the
     weights and ``topk_scores``)."""
-    p = get_token_indices(topk_indices, topk, num_experts, zero_prefix=True)
+    with scope("get_token_indices"):
+        p = get_token_indices(topk_indices, topk, num_experts, zero_prefix=True)
     return _ExpertsFunction.apply(x, weight1, weight2, topk_scores, p.group_indices, p.indices,
                                   activation_name(act), topk)
 
 
+def shared_experts(input, sp):
+    """The reference's shared-expert branch (``topk_moe.py:56-62``): every token through each
+    of the S shared FFNs, summed over S (its ``h.sum(0)`` over stacked ``[S, d, ff]`` /
+    ``[S, ff, d]`` weights; 2-D weights are one shared expert).  Runs on the grouped-GEMM
+    kernels as S experts that every token is routed to with weight 1, so the forward is two
+    grouped GEMMs and the backward the routed experts' own."""
+    up, down = sp.up_weight, sp.down_weight
+    if up.dim() == 2:
+        up, down = up.unsqueeze(0), down.unsqueeze(0)
+    assert up.dim() == 3 and down.dim() == 3 and up.size(0) == down.size(0)
+    S, T = up.size(0), input.size(0)
+    ones = torch.ones((T, S), device=input.device, dtype=input.dtype)
+    ids = torch.arange(S, device=input.device, dtype=torch.int64).expand(T, S)
+    return routed_experts(input, up, down, ones, ids, S, S, sp.activation)
+
+
 def topk_moe_forward(input: torch.Tensor, params: MOEParams, autotune_mode=None):
     w1, w2, act = expert_weights(params.expert_params)
-    topk_scores, topk_indices = router(input, params.router_params)
+    with scope("router"):
+        topk_scores, topk_indices = router(input, params.router_params)
     out = routed_experts(input, w1, w2, topk_scores, topk_indices, params.num_experts,
                          params.topk, act)
-    sp = params.shared_expert_params
+    sp = getattr(params, "shared_expert_params", None)
     if sp is not None:
-        # intended form of the reference's shared-expert branch (topk_moe.py:56-62):
-        # a dense FFN applied to every token and added to the routed output
-        hid = activation(input @ sp.up_weight, sp.activation)
-        out = out + hid @ sp.down_weight
+        with scope("shared_expert"):
+            out = out + shared_experts(input, sp)
     return out
 
 

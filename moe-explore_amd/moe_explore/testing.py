@@ -61,6 +61,27 @@ def random_skewed_routing(num_tokens, num_experts, topk, num_skewed_experts, ske
     return topk_scores, topk_indices
 
 
+# Share (in percent, top-8) of tokens that reach each of OLMoE-1B-7B's 64 experts in the layer
+# the reference measured (the table embedded in ``testing.py:141-206``, rounded to 1e-3).
+OLMOE_EXPERT_LOAD_PERCENT = (
+    18.016, 16.976, 12.5, 10.182, 7.372, 15.966, 9.168, 11.66, 15.418, 17.458, 10.972, 12.994,
+    9.004, 17.926, 13.156, 10.016, 8.604, 21.036, 8.512, 3.96, 2.616, 6.664, 8.37, 16.756, 18.186,
+    2.848, 7.324, 8.522, 9.532, 8.648, 12.092, 24.614, 15.37, 7.922, 13.118, 2.748, 16.314, 19.992,
+    9.774, 13.298, 37.532, 16.268, 7.85, 12.164, 18.804, 10.76, 7.862, 19.14, 6.974, 13.958, 9.122,
+    8.742, 12.018, 16.918, 26.756, 8.796, 4.726, 16.596, 7.27, 11.458, 9.91, 6.098, 26.756, 8.686,
+)
+
+
+def random_olmoe_routing(num_tokens, num_experts, topk, device, dtype):
+    """Experts drawn without replacement with OLMoE's measured per-expert loads as weights
+    (``testing.py:134-209``); 64 experts only, as there."""
+    assert num_experts == len(OLMOE_EXPERT_LOAD_PERCENT), "the load table has 64 experts"
+    probabilities = torch.tensor(OLMOE_EXPERT_LOAD_PERCENT, device=device, dtype=torch.float32) / 100.0
+    topk_indices = torch.multinomial(probabilities.repeat(num_tokens, 1), num_samples=topk, replacement=False)
+    topk_scores, _ = random_routing(num_tokens, num_experts, topk, device, dtype)
+    return topk_scores, topk_indices
+
+
 def random_zipf_routing(num_tokens, num_experts, topk, device, dtype, s=1.2, generator=None):
     """Top-k of normal logits plus ``log p_e`` with ``p_e`` Zipf(s) over a random
     permutation of the experts: a few heavy experts and some near-empty ones."""

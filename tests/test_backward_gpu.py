@@ -88,6 +88,28 @@ def test_k_grouped_gemm_many_uneven_experts():
             assert_parity(out[e], ref[e], torch.bfloat16, f"expert {e}")
 
 
+@pytest.mark.parametrize("E,Ka,Nb", [(160, 264, 520), (200, 520, 776)])
+def test_k_grouped_gemm_more_experts_than_the_balanced_deal_takes(E, Ka, Nb):
+    """More than 128 uneven experts (and, second case, more than 512 chunks of tiles): the
+    kernel keeps its round-robin deal of tile chunks instead of the one balanced by load."""
+    from moe_explore.triton_kernels.m_grouped_gemm import k_grouped_gemm
+    sizes = [max(0, int(1500 / (i + 1) ** 1.1) - 5) for i in range(E)]
+    sizes = [sizes[(53 * i) % E] for i in range(E)]
+    g = seeded(E)
+    rows = sum(sizes)
+    gi = torch.zeros(E + 1, dtype=torch.int32)
+    gi[1:] = torch.cumsum(torch.tensor(sizes), 0)
+    a, b = randn((rows, Ka), g, torch.bfloat16), randn((rows, Nb), g, torch.bfloat16)
+    out = k_grouped_gemm(a.cuda(), b.cuda(), gi.cuda())
+    ref = moe_ref.k_grouped_matmul(a, b, gi)
+    assert_parity(out, ref, torch.bfloat16, f"k_grouped_gemm, {E} uneven experts")
+    for e in range(E):
+        if sizes[e] == 0:
+            assert (out[e] == 0).all()
+        elif e % 7 == 0 or sizes[e] < 4:
+            assert_parity(out[e], ref[e], torch.bfloat16, f"expert {e} ({sizes[e]} rows)")
+
+
 @pytest.mark.parametrize("which", ["a", "b"])
 def test_k_grouped_gemm_gather(which):
     from moe_explore.expert_permute import get_token_indices
@@ -224,9 +246,9 @@ def test_layer_backward(T, d, ff, E, k, act, dtype):
 
 
 def test_backward_config1_properties():
-    """BASELINE config 1 (d_ff reduced 8x so the autograd oracle runs in seconds) on a
-    token subset is not possible for dW (it sums over all tokens), so the full-width
-    check uses fewer tokens per expert instead: T=1024."""
+    """BASELINE config 1 with d_ff reduced 8x and T=1024, so that autograd through the
+    oracle covers every element of every gradient in seconds (the full size is checked on
+    token and column subsets in test_backward_configs_gpu.py)."""
     from moe_explore.functional.topk_moe import routed_experts
     g = seeded(8)
     T, d, ff, E, k = 1024, 1024, 1792, 8, 2

@@ -118,3 +118,68 @@ def test_fp8_full_size_t8192_runs_and_is_linear_in_scores():
     half = routed_experts_fp8(x, params, scores * 0.5, idx, E, k)
     assert torch.isfinite(out.float()).all()
     assert torch.equal(half.float() * 2, out.float())
+
+
+@pytest.fixture(scope="module")
+def config4_weights():
+    """Config-4 weights at full width (d=4096, ff=14336, E=8): N(0, 0.02) bf16 made on the GPU,
+    their fp8 quantisation, and an fp32 copy on the host for the oracle."""
+    dev = "cuda"
+    gd = torch.Generator(device=dev).manual_seed(4)
+    d, ff, E = 4096, 14336, 8
+    w1 = torch.empty((E, d, 2 * ff), device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=gd)
+    w2 = torch.empty((E, ff, d), device=dev, dtype=torch.bfloat16).normal_(0, 0.02, generator=gd)
+    from moe_explore.fp8 import quantize_expert_weights
+    q1, q2 = quantize_expert_weights(w1), quantize_expert_weights(w2)
+    host = (w1.cpu().float(), w2.cpu().float())
+    del w1, w2
+    torch.cuda.empty_cache()
+    yield q1, q2, host
+    del q1, q2, host
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("T,checked", [(128, 32), (1024, 48)])
+@pytest.mark.parametrize("act", ["swiglu", "geglu"])
+def test_fp8_layer_full_width_against_bf16_weights(config4_weights, T, checked, act):
+    """Config 4 at its real width, T = 128 and 1024 (the weight-streaming regime: split-K down
+    projection, tile-major weights): the fp8 layer against the fp32 oracle on the unquantised
+    weights for a subset of tokens (a token's output depends on its own row), <= 8e-2."""
+    from moe_explore.fp8 import Fp8MLPParams, routed_experts_fp8
+    q1, q2, (w1, w2) = config4_weights
+    g = seeded(T + len(act))
+    d, E, k = 4096, 8, 2
+    x = randn((T, d), g, torch.bfloat16)
+    scores, idx = moe_ref.route_from_logits(torch.randn((T, E), generator=g), k, True, True, torch.bfloat16)
+    out = routed_experts_fp8(x.cuda(), Fp8MLPParams(q1, q2, act), scores.cuda(), idx.cuda(), E, k)
+    assert torch.isfinite(out.float()).all()
+    sel = torch.randperm(T, generator=g)[:checked]
+    ref = moe_ref.experts_forward(x[sel], w1, w2, scores[sel], idx[sel], E, k, act)
+    err = moe_ref.rel_fro(out[sel.cuda()], ref)
+    assert err <= 8e-2, f"fp8 layer, T={T}, {act}: rel-Frobenius {err:.3e} vs the bf16-weight oracle"
+
+
+@pytest.mark.parametrize("T", [128, 1024])
+def test_fp8_gate_up_gemm_full_width_against_dequantised_oracle(config4_weights, T):
+    """The gate/up fp8 GEMM alone at full width (N = 28672, tile-major weights) against fp32
+    products of the SAME codes and scales: rows of two experts, every column."""
+    from moe_explore.expert_permute import get_token_indices
+    from moe_explore.fp8 import m_grouped_gemm_fp8, quantize_rows
+    q1, _, _ = config4_weights
+    g = seeded(T)
+    d, E, k = 4096, 8, 2
+    x = randn((T, d), g, torch.bfloat16)
+    _, idx = moe_ref.route_from_logits(torch.randn((T, E), generator=g), k, True, True, torch.bfloat16)
+    p = get_token_indices(idx.cuda(), k, E, zero_prefix=True)
+    xq, xs = quantize_rows(x.cuda())
+    h = m_grouped_gemm_fp8(xq, xs, q1, p.group_indices, p.indices, gather=True, num_tokens=T, topk=k)
+    gi, ind = p.group_indices.cpu(), p.indices.cpu()
+    xd = xq.cpu().float() * xs.cpu().unsqueeze(1)
+    for e in (0, E - 1):
+        lo, hi = int(gi[e]), min(int(gi[e + 1]), int(gi[e]) + 24)
+        if hi <= lo:
+            continue
+        codes = q1.codes()[e]                                        # [N, K] on the GPU
+        wd = (codes.float() * q1.scale[e].unsqueeze(-1)).t().cpu()   # [K, N]
+        ref = xd[ind[lo:hi] // k] @ wd
+        assert_parity(h[lo:hi], ref, torch.bfloat16, f"fp8 gate/up GEMM, expert {e}", tol=1e-2)

@@ -82,3 +82,53 @@ def test_testing_helpers():
     testing.assert_close(a, a.clone())
     with pytest.raises(AssertionError):
         testing.assert_close(a, a + 1)
+
+
+@pytest.mark.parametrize("gather,scatter,act", [(False, False, None), (True, False, "swiglu"),
+                                                (False, True, None), (False, False, "gelu")])
+def test_package_op_level_loop_matches_the_oracle(gather, scatter, act):
+    """moe_explore.testing.torch_grouped_matmul_gather_scatter (the reference's comparison
+    implementation, testing.py:9-50, as the package ships it) against the oracle's."""
+    from moe_explore.testing import torch_grouped_matmul_gather_scatter
+    from moe_explore.triton_kernels.m_grouped_gemm import MGroupedGEMMParams
+    from oracle import moe_ref
+    g = seeded(5)
+    T, E, k, K, N = 40, 4, 2, 16, 24
+    _, idx = moe_ref.route_from_logits(torch.randn((T, E), generator=g), k)
+    gi, ind = moe_ref.get_token_indices(idx, k, E, zero_prefix=True)
+    rows = T if gather else T * k
+    a = torch.randn((rows, K), generator=g)
+    w = torch.randn((E, K, N), generator=g)
+    scales = torch.rand((T, k), generator=g) if scatter else None
+    p = MGroupedGEMMParams(w, gi, ind if (gather or scatter) else None, gather, scatter,
+                           T if (gather or scatter) else rows, k, scales=scales, activation=act)
+    out = torch_grouped_matmul_gather_scatter(a, p)
+    ref = moe_ref.grouped_matmul_gather_scatter(a, w, gi, p.permute_indices, gather, scatter, T, k,
+                                                scales, act)
+    torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
+
+
+def test_interleaved_copy_of_separate_gate_up_weights_is_cached_on_cpu():
+    from moe_explore.functional import topk_moe as layer
+    from moe_explore.params import GLUParams
+    g = seeded(6)
+    gate, up, down = (torch.randn(s, generator=g) for s in ((3, 8, 6), (3, 8, 6), (3, 6, 8)))
+    ep = GLUParams(gate, up, down, "swiglu")
+    w_a = layer.expert_weights(ep)[0]
+    assert layer.expert_weights(ep)[0] is w_a
+    assert torch.equal(w_a[..., 0::2], gate) and torch.equal(w_a[..., 1::2], up)
+    up.add_(1.0)                                      # written: the copy is rebuilt
+    w_b = layer.expert_weights(ep)[0]
+    assert w_b is not w_a and torch.equal(w_b[..., 1::2], up)
+    gate.requires_grad_(True)
+    w_c = layer.expert_weights(ep)[0]
+    w_c.sum().backward()
+    assert torch.equal(gate.grad, torch.ones_like(gate))
+    assert layer.to_interleaved(ep).interleaved_weight.shape == (3, 8, 12)
+
+
+def test_stage_ranges_are_off_by_default_and_nest():
+    from moe_explore import tracing
+    assert not tracing.enabled()
+    with tracing.scope("router"):
+        pass

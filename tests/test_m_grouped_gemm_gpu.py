@@ -304,3 +304,108 @@ def test_launches_on_two_streams_do_not_share_tile_counters():
     torch.cuda.synchronize()
     for s in range(2):
         assert torch.equal(outs[s], serial[s]), f"stream {s}"
+
+
+def _graph_of(fn, warmups=2):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(warmups):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fn()
+    return graph, out
+
+
+def test_captured_launches_own_no_tile_counters():
+    """A launch recorded into a HIP graph takes its tile ids in strides of the grid instead of
+    from a queue set, so replays share no device state with anything: two graphs of the same
+    GEMM replayed on two streams at once, next to eager launches of it on a third and fourth,
+    all give the serial result; and a graph captured before 1500 eager launches (more than
+    there are queue sets) still replays bit-exactly afterwards."""
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    g = seeded(79)
+    T, E, K, N = 5000, 4, 512, 1024
+    x = randn((T, K), g, torch.bfloat16).cuda()
+    w = randn((E, K, N), g, torch.bfloat16, 1.0 / math.sqrt(N)).cuda()
+    gi = random_group_indices(T, E, g).cuda()
+    p = _params(w, gi, None, False, False, T, 1, activation="swiglu")
+    with torch.no_grad():
+        serial = m_grouped_gemm(x, p).clone()
+        graphs = [_graph_of(lambda: m_grouped_gemm(x, p)) for _ in range(2)]
+        torch.cuda.synchronize()
+        streams = [torch.cuda.Stream() for _ in range(4)]
+        eager = [torch.empty_like(serial) for _ in range(2)]
+        for rep in range(10):
+            for i, (graph, out) in enumerate(graphs):
+                with torch.cuda.stream(streams[i]):
+                    graph.replay()
+            for i in range(2):
+                with torch.cuda.stream(streams[2 + i]):
+                    m_grouped_gemm(x, p, out=eager[i])
+            if rep % 3 == 2:
+                torch.cuda.synchronize()
+                for i, (_, out) in enumerate(graphs):
+                    assert torch.equal(out, serial), f"graph {i}, round {rep}"
+                    out.fill_(float("nan"))
+                for i in range(2):
+                    assert torch.equal(eager[i], serial), f"eager stream {i}, round {rep}"
+        torch.cuda.synchronize()
+        # many eager launches later the first graph is still good
+        scratch = torch.empty_like(serial)
+        for _ in range(1500):
+            m_grouped_gemm(x, p, out=scratch)
+        graph, out = graphs[0]
+        out.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, serial) and torch.equal(scratch, serial)
+
+
+def test_many_streams_each_get_a_queue_set():
+    """Eager launches on 24 streams in flight together."""
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    g = seeded(80)
+    T, E, K, N = 3000, 4, 256, 512
+    x = randn((T, K), g, torch.bfloat16).cuda()
+    w = randn((E, K, N), g, torch.bfloat16, 1.0 / math.sqrt(N)).cuda()
+    gi = random_group_indices(T, E, g).cuda()
+    p = _params(w, gi, None, False, False, T, 1, activation=None)
+    serial = m_grouped_gemm(x, p).clone()
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(24)]
+    outs = [torch.empty_like(serial) for _ in streams]
+    for rep in range(5):
+        for s, o in zip(streams, outs):
+            with torch.cuda.stream(s):
+                m_grouped_gemm(x, p, out=o)
+    torch.cuda.synchronize()
+    for i, o in enumerate(outs):
+        assert torch.equal(o, serial), f"stream {i}"
+
+
+def test_split_k_with_transposed_weights():
+    """ksplit = 2 on the K-contiguous (transposed) weight view, the form the dX GEMM of the
+    backward pass runs at K = 2 * d_ff; the two partial products add up to the unsplit one."""
+    from moe_explore.functional.scale_and_reduce import scale_and_reduce
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    g = seeded(81)
+    T, E, K, N, topk = 1536, 4, 1024, 512, 2
+    R = T * topk
+    a = randn((R, K), g, torch.bfloat16).cuda()
+    w = randn((E, N, K), g, torch.bfloat16, 1.0 / math.sqrt(K)).cuda()      # [E, N, K]: used as w^T
+    gi = random_group_indices(R, E, g).cuda()
+    perm = torch.randperm(R, generator=g).cuda()
+    p = _params(w, gi, perm, False, True, T, topk)
+    whole = m_grouped_gemm(a, p, transpose_weight=True)
+    parts = m_grouped_gemm(a, p, transpose_weight=True, ksplit=2)
+    assert parts.shape == (2 * R, N), "the split was declined"
+    ref = moe_ref.grouped_matmul_gather_scatter(a.cpu(), w.transpose(1, 2).cpu(), gi.cpu(), perm.cpu(),
+                                                scatter=True, num_tokens=T, topk=topk)
+    assert_parity(parts[:R].float() + parts[R:].float(), ref, torch.bfloat16, "sum of the K parts")
+    assert_parity(whole, ref, torch.bfloat16, "unsplit")
+    summed = scale_and_reduce(parts, None, T, topk, N, nsplit=2)
+    want = ref.view(T, topk, N).sum(1)
+    assert_parity(summed, want, torch.bfloat16, "scale_and_reduce over parts and top-k")

@@ -147,6 +147,10 @@ def test_router_backward_matches_autograd(mode, dtype):
     # oracle: fp32 autograd through the same formulas with the same selection
     xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
     logits = xr @ wr
+    if mode != "ernie":
+        # the reference's matmul returns the logits in the dtype of x (router.py:22); rounding
+        # has no gradient of its own (straight through)
+        logits = logits + (logits.to(dtype).float() - logits).detach()
     if mode == "topk_first":
         sr = torch.softmax(torch.gather(logits, 1, idx), -1)
     else:
@@ -156,7 +160,7 @@ def test_router_backward_matches_autograd(mode, dtype):
         elif mode == "ernie":
             sr = sr / sr.sum(-1, keepdim=True).clamp_min(1e-12)
     sr.backward(g.float())
-    tol = 1e-4 if dtype == torch.float32 else 3e-2
+    tol = 1e-4 if dtype == torch.float32 else 2e-2   # the bar for bf16 results
     assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= tol
     assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= tol
 
