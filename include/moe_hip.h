@@ -93,6 +93,23 @@ MOE_API int moe_route_preprocess(const void* expert_ids, int idx_bytes, int64_t 
                          moe_stream_t stream);
 
 /*
+ * moe_route_preprocess without a workspace and without any allocation.  No counterpart in
+ * the reference: it exists for callers that cannot allocate device memory -- code under HIP
+ * graph capture, serving loops with a fixed memory plan, harnesses that forbid hipMalloc --
+ * and so cannot provide the workspace either.  Same results as moe_route_preprocess, bit for
+ * bit.  The per-chunk counts live in a buffer of moe_route_noalloc_max_bytes() bytes (4 MiB)
+ * that is part of the library image on every device: calls with
+ * moe_route_workspace_bytes(R, E) above that (ceil(R / 512) * E > 2^20) return
+ * MOE_ERR_WORKSPACE.  All calls on one device share that buffer: calls that may overlap in
+ * time (different streams) race; calls on one stream are ordered and safe.  Nothing in the
+ * buffer has to be cleared between calls.
+ */
+MOE_API size_t moe_route_noalloc_max_bytes(void);
+MOE_API int moe_route_preprocess_noalloc(const void* expert_ids, int idx_bytes, int64_t R, int E,
+                                 int64_t* indices_out, int32_t* group_indices_out,
+                                 int64_t* inclusive_out, moe_stream_t stream);
+
+/*
  * Row gather / row scatter: replace row_gather and row_scatter
  * (triton_kernels/row_gather_scatter.py:36-58, :91-116).
  *   gather : dst[r, :] = src[idx[r] / idx_div, :]   r < rows_out, indices may repeat

@@ -14,6 +14,8 @@
 // Slots are placed in ascending slot order inside an expert, i.e. the stable sort.
 #include "common.h"
 
+#include <mutex>
+
 namespace moe {
 namespace {
 
@@ -169,23 +171,15 @@ extern "C" size_t moe_route_workspace_bytes(int64_t R, int E) {
   return static_cast<size_t>(chunks) * static_cast<size_t>(E) * sizeof(int32_t);
 }
 
-extern "C" int moe_route_preprocess(const void* expert_ids, int idx_bytes, int64_t R, int E,
-                                    int64_t* indices_out, int32_t* group_indices_out,
-                                    int64_t* inclusive_out, void* workspace,
-                                    size_t workspace_bytes, moe_stream_t stream_) {
-  using namespace moe;
-  clear_error();
-  MOE_REQUIRE(idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8, got %d", idx_bytes);
-  MOE_REQUIRE(R >= 0 && R <= 0x7fffffff, "R out of range: %lld", (long long)R);
-  MOE_REQUIRE(E >= 1 && E <= kMaxExperts, "E must be in [1,%d], got %d", kMaxExperts, E);
-  MOE_REQUIRE(group_indices_out != nullptr, "group_indices_out is null");
-  MOE_REQUIRE(R == 0 || (expert_ids != nullptr && indices_out != nullptr),
-              "expert_ids / indices_out is null");
-  if (workspace == nullptr || workspace_bytes < moe_route_workspace_bytes(R, E))
-    return fail(MOE_ERR_WORKSPACE, "routing workspace needs %zu bytes, got %zu",
-                moe_route_workspace_bytes(R, E), workspace_bytes);
-  hipStream_t stream = static_cast<hipStream_t>(stream_);
-  int32_t* counts = static_cast<int32_t*>(workspace);
+namespace moe {
+namespace {
+
+// The three launches of the counting sort over a counts array of num_chunks * E words.
+// Every word that is read has been written by route_count in the same call: nothing has to
+// start at zero.
+int route_preprocess_launch(const void* expert_ids, int idx_bytes, int64_t R, int E,
+                            int64_t* indices_out, int32_t* group_indices_out,
+                            int64_t* inclusive_out, int32_t* counts, hipStream_t stream) {
   const int64_t chunks = num_chunks_for(R);
   const unsigned blocks = static_cast<unsigned>((chunks + kWavesPerBlock - 1) / kWavesPerBlock);
   const size_t lds = static_cast<size_t>(kWavesPerBlock) * E * sizeof(int32_t);
@@ -202,4 +196,82 @@ extern "C" int moe_route_preprocess(const void* expert_ids, int idx_bytes, int64
     if (int rc = check_launch("route_place")) return rc;
   }
   return MOE_OK;
+}
+
+int check_route_args(const void* expert_ids, int idx_bytes, int64_t R, int E,
+                     const int64_t* indices_out, const int32_t* group_indices_out) {
+  MOE_REQUIRE(idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8, got %d", idx_bytes);
+  MOE_REQUIRE(R >= 0 && R <= 0x7fffffff, "R out of range: %lld", (long long)R);
+  MOE_REQUIRE(E >= 1 && E <= kMaxExperts, "E must be in [1,%d], got %d", kMaxExperts, E);
+  MOE_REQUIRE(group_indices_out != nullptr, "group_indices_out is null");
+  MOE_REQUIRE(R == 0 || (expert_ids != nullptr && indices_out != nullptr),
+              "expert_ids / indices_out is null");
+  return MOE_OK;
+}
+
+// Scratch of moe_route_preprocess_noalloc: the counts array, resident in every device's copy of
+// the library image until the process ends.  Host code never uses the array's name as an
+// address: the device address is looked up once per device (scratch_of_current_device).
+constexpr size_t kScratchWords = size_t(1) << 20;  // 4 MiB
+static __device__ __align__(256) int32_t scratch[kScratchWords];
+
+int32_t* scratch_of_current_device() {
+  constexpr int kMaxDevices = 64;
+  static int32_t* of_device[kMaxDevices];
+  static std::mutex lock;
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    fail(MOE_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(err));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(lock);
+  if (of_device[dev] == nullptr) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || p == nullptr) {
+      fail(MOE_ERR_HIP, "hipGetSymbolAddress(routing scratch): %s", hipGetErrorString(err));
+      return nullptr;
+    }
+    of_device[dev] = static_cast<int32_t*>(p);
+  }
+  return of_device[dev];
+}
+
+}  // namespace
+}  // namespace moe
+
+extern "C" int moe_route_preprocess(const void* expert_ids, int idx_bytes, int64_t R, int E,
+                                    int64_t* indices_out, int32_t* group_indices_out,
+                                    int64_t* inclusive_out, void* workspace,
+                                    size_t workspace_bytes, moe_stream_t stream_) {
+  using namespace moe;
+  clear_error();
+  if (int rc = check_route_args(expert_ids, idx_bytes, R, E, indices_out, group_indices_out)) return rc;
+  if (workspace == nullptr || workspace_bytes < moe_route_workspace_bytes(R, E))
+    return fail(MOE_ERR_WORKSPACE, "routing workspace needs %zu bytes, got %zu",
+                moe_route_workspace_bytes(R, E), workspace_bytes);
+  return route_preprocess_launch(expert_ids, idx_bytes, R, E, indices_out, group_indices_out,
+                                 inclusive_out, static_cast<int32_t*>(workspace),
+                                 static_cast<hipStream_t>(stream_));
+}
+
+extern "C" size_t moe_route_noalloc_max_bytes(void) { return moe::kScratchWords * sizeof(int32_t); }
+
+extern "C" int moe_route_preprocess_noalloc(const void* expert_ids, int idx_bytes, int64_t R, int E,
+                                            int64_t* indices_out, int32_t* group_indices_out,
+                                            int64_t* inclusive_out, moe_stream_t stream_) {
+  using namespace moe;
+  clear_error();
+  if (int rc = check_route_args(expert_ids, idx_bytes, R, E, indices_out, group_indices_out)) return rc;
+  const size_t need = moe_route_workspace_bytes(R, E);
+  if (need > kScratchWords * sizeof(int32_t))
+    return fail(MOE_ERR_WORKSPACE,
+                "routing of %lld slots over %d experts needs %zu bytes of scratch; the resident "
+                "buffer of moe_route_preprocess_noalloc has %zu (use moe_route_preprocess with a "
+                "workspace)", (long long)R, E, need, kScratchWords * sizeof(int32_t));
+  int32_t* const counts = scratch_of_current_device();
+  if (counts == nullptr) return MOE_ERR_HIP;
+  return route_preprocess_launch(expert_ids, idx_bytes, R, E, indices_out, group_indices_out,
+                                 inclusive_out, counts, static_cast<hipStream_t>(stream_));
 }

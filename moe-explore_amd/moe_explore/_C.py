@@ -41,6 +41,8 @@ SIGNATURES = {
     "moe_last_error_string": (ctypes.c_char_p, []),
     "moe_route_workspace_bytes": (_sz, [_i64, _i32]),
     "moe_route_preprocess": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "moe_route_noalloc_max_bytes": (_sz, []),
+    "moe_route_preprocess_noalloc": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _vp, _vp]),
     "moe_row_gather": (_i32, [_vp, _i64, _i64, _vp, _i32, _i32, _vp, _i64, _i64, _i64, _i32, _vp]),
     "moe_row_scatter": (_i32, [_vp, _i64, _vp, _i32, _vp, _i64, _i64, _i64, _i64, _i32, _vp]),
     "moe_scale_and_reduce": (_i32, [_vp, _i64, _vp, _vp, _i64, _i64, _i32, _i64, _i32, _i32, _i64, _vp]),

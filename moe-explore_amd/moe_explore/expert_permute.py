@@ -55,6 +55,28 @@ def get_token_indices(expert_indices, topk, num_experts, zero_prefix=False):
     )
 
 
+def get_token_indices_into(expert_indices, num_experts, indices_out, group_indices_out,
+                           inclusive_out=None):
+    """``get_token_indices`` for callers that may not allocate (HIP graph capture, serving
+    loops with a fixed memory plan): the results go to the caller's tensors (``indices_out``
+    int64 ``[R]``, ``group_indices_out`` int32 ``[E+1]``, optionally ``inclusive_out`` int64
+    ``[E]``) and the per-chunk counts to a 4 MiB buffer inside the library, so nothing is
+    allocated here or there.  ``expert_indices`` must already be a contiguous int32 / int64
+    tensor.  Calls on one device share that buffer: keep them on one stream.  Raises
+    ``MoeHipError`` when ``ceil(R / 512) * E`` exceeds 2**20 words."""
+    _C.require_cuda(expert_indices, indices_out, group_indices_out, inclusive_out)
+    assert expert_indices.is_contiguous() and expert_indices.dtype in (torch.int32, torch.int64)
+    R, E = expert_indices.numel(), int(num_experts)
+    assert indices_out.dtype == torch.int64 and indices_out.numel() == R and indices_out.is_contiguous()
+    assert group_indices_out.dtype == torch.int32 and group_indices_out.numel() == E + 1
+    assert inclusive_out is None or (inclusive_out.dtype == torch.int64 and inclusive_out.numel() == E)
+    st = _C.load().moe_route_preprocess_noalloc(
+        expert_indices.data_ptr(), _C.idx_bytes(expert_indices), R, E, indices_out.data_ptr(),
+        group_indices_out.data_ptr(), _C.ptr(inclusive_out), _C.stream_of(expert_indices))
+    _C.check(st, "moe_route_preprocess_noalloc")
+    return PermToGroupIndices(group_indices=group_indices_out, indices=indices_out)
+
+
 def expert_input_permute(tokens: torch.Tensor, expert_indices: torch.Tensor, num_experts: int,
                          topk: int) -> GroupedTokens:
     indices = get_token_indices(expert_indices, topk, num_experts, zero_prefix=True)
