@@ -45,6 +45,35 @@ def make_inputs(cfg, device, seed=0):
     return x, w1, w2, wr, dout
 
 
+PROFILE_OF_DOMINANT_KERNEL = os.path.join(ROOT, "profiles", "m_grouped_dma_kernel_mixtral_config1.txt")
+KERNEL_SOURCES = [os.path.join(ROOT, "moe-explore_amd", "csrc", f) for f in ("gemm_mfma_dma.hip", "gemm_mfma.h")]
+
+
+def kernel_source_digest():
+    """sha256 (first 16 hex digits) over the sources of the dominant kernel."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in KERNEL_SOURCES:
+        with open(path, "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profiled_traffic_bytes():
+    """HBM bytes a launch of the dominant kernel from the tracked rocprofv3 summary (its line
+    `TRAFFIC_BYTES_PER_LAUNCH=... KERNEL_SOURCE_SHA256_16=...`), or None when the summary is
+    missing or was made from other kernel sources than the ones in the tree."""
+    import re
+    try:
+        text = open(PROFILE_OF_DOMINANT_KERNEL).read()
+    except OSError:
+        return None
+    m = re.search(r"TRAFFIC_BYTES_PER_LAUNCH=([0-9.eE+]+)\s+KERNEL_SOURCE_SHA256_16=([0-9a-f]{16})", text)
+    if not m or m.group(2) != kernel_source_digest():
+        return None
+    return float(m.group(1))
+
+
 def device_clock_mhz():
     """Maximum shader clock of the first GPU agent that rocminfo lists (0.0 if it cannot be
     read); run as a child process."""
@@ -96,7 +125,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--mode", choices=["fwdbwd", "fwd"], default="fwdbwd")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23"],
+    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23", "fp8", "digest"],
                     default="all",
                     help="profiling aids: 'kernel' launches only the dominant GEMM --steps times, "
                          "'copy' only a 1 GiB device copy (the known-size kernel that calibrates "
@@ -106,13 +135,19 @@ def main():
                          "combine) at the shapes of configs 1-3 with their algorithmic bytes and "
                          "event-timed GB/s, 'configs23' the routed experts (forward, then forward + "
                          "backward) at the shapes of configs 2 and 3, config 3 with Zipf(1.2) expert "
-                         "loads; none of them prints the JSON line")
+                         "loads, 'fp8' the fp8 inference layer (config 4: T = 128, 1024, 8192, GeGLU) "
+                         "with its weight-streaming rate and TFLOP/s, 'digest' prints the digest of "
+                         "the dominant kernel's sources that a profile summary records; none of "
+                         "them prints the JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1",
               file=sys.stderr)
         sys.exit(2)
 
+    if args.only == "digest":
+        print("KERNEL_SOURCE_SHA256_16=" + kernel_source_digest())
+        return
     import torch
     from moe_explore import _C
     from moe_explore.expert_permute import get_token_indices
@@ -131,6 +166,32 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print("copied 1 GiB x %d" % args.steps)
+        return
+    if args.only == "fp8":
+        from moe_explore.fp8 import Fp8MLPParams, quantize_expert_weights, routed_experts_fp8
+        from moe_explore.router import route_from_logits
+        d, ff, E, k = cfg["d"], cfg["ff"], cfg["E"], cfg["k"]
+        gd = torch.Generator(device=dev).manual_seed(0)
+        w1 = torch.empty((E, d, 2 * ff), device=dev, dtype=torch.bfloat16).normal_(0.0, 0.02, generator=gd)
+        w2 = torch.empty((E, ff, d), device=dev, dtype=torch.bfloat16).normal_(0.0, 0.02, generator=gd)
+        params = Fp8MLPParams(quantize_expert_weights(w1), quantize_expert_weights(w2), "geglu")
+        del w1, w2
+        weight_bytes = 3.0 * E * d * ff      # e4m3: one byte a weight
+        for T in (128, 1024, 8192):
+            x = torch.randn((T, d), device=dev, generator=gd).to(torch.bfloat16)
+            scores, idx = route_from_logits(torch.randn((T, E), device=dev, generator=gd), k, True, True,
+                                            torch.bfloat16)
+            with torch.no_grad():
+                for _ in range(args.warmup):
+                    routed_experts_fp8(x, params, scores, idx, E, k)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    routed_experts_fp8(x, params, scores, idx, E, k)
+                torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) / args.steps * 1e3
+            print("fp8 layer fwd (geglu) T=%5d: %7.3f ms  %7.1f TFLOP/s  weights streamed at %6.0f GB/s" % (
+                T, ms, 6.0 * T * k * d * ff / ms / 1e9, weight_bytes / ms / 1e6), flush=True)
         return
     if args.only == "router":
         from moe_explore.router import route_from_logits
@@ -333,8 +394,9 @@ def main():
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "launch_ms": round(k_ms, 4), "flops_per_launch": k_flops,
                      # HBM bytes a launch from rocprofv3 FETCH_SIZE / WRITE_SIZE, calibrated
-                     # with a 1 GiB copy (profiles/m_grouped_dma_kernel_mixtral_config1.txt)
-                     "traffic": 7.63e9},
+                     # with a 1 GiB copy, read from the tracked summary of that profile; null
+                     # when the kernel's sources have changed since it was made
+                     "traffic": profiled_traffic_bytes()},
         # peak recomputed from what the device reports; the sustained clock under this load
         # is lower (about 1.65-1.8 GHz with random operands)
         "device": {"name": props.name, "cus": props.multi_processor_count, "clock_mhz": clock_mhz,
