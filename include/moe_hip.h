@@ -66,6 +66,8 @@ typedef void* moe_stream_t;
 /* flags of moe_k_grouped_gemm */
 #define MOE_KGEMM_GATHER_A 1 /* A row of position p is a[indices[p] / topk] */
 #define MOE_KGEMM_GATHER_B 2 /* B row of position p is b[indices[p] / topk] */
+#define MOE_KGEMM_A_KMAJOR 4 /* a is [Ka, columns], written by moe_row_gather_kmajor */
+#define MOE_KGEMM_B_KMAJOR 8 /* b is [Nb, columns], written by moe_row_gather_kmajor */
 
 /* Library version: major*10000 + minor*100 + patch. */
 MOE_API int moe_version(void);
@@ -188,7 +190,26 @@ MOE_API int moe_m_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, const
  *              a[arow(p), :]^T (outer) b[brow(p), :]          fp32 accumulate
  *   a [*, Ka], b [*, Nb] in `dtype` (row strides lda, ldb); out [E, Ka, Nb] in
  *   `dtype`, contiguous.  Experts with no rows get zeros.
+ * MOE_KGEMM_A_KMAJOR / MOE_KGEMM_B_KMAJOR (one of them, no gather flags): that operand is
+ * given feature-major, [Ka or Nb, columns] with row stride lda / ldb and a_rows / b_rows
+ * counting its columns (>= moe_kmajor_columns(P, E)), in the layout moe_row_gather_kmajor
+ * writes.  The weight gradients' small operand is a set of gathered token rows that has
+ * to be materialised anyway; feature-major, the kernel reads it from LDS with plain
+ * 16-byte loads instead of transpose loads (16-bit dtypes, MFMA kernel only:
+ * MOE_ERR_UNSUPPORTED otherwise).
+ *
+ * moe_row_gather_kmajor: dst[f, qs(e) + (p - lo(e))] = src[idx[p] / idx_div, f] for every
+ * position p of expert e (lo(e) = group_indices[e]), where qs(e) = 64 * (lo(e) / 64 + e):
+ * every expert's segment starts on a multiple of 64 columns and is followed by zeros up to
+ * the next multiple of 64.  dst is [features, ld_dst] with ld_dst >= moe_kmajor_columns(P, E)
+ * = 64 * (P / 64 + E + 1); columns outside the segments and their zero fill are not written.
+ * No counterpart in the reference (forward-only).
  */
+MOE_API int64_t moe_kmajor_columns(int64_t P, int E);
+MOE_API int moe_row_gather_kmajor(const void* src, int64_t src_rows, int64_t src_stride,
+                          const void* idx, int idx_bytes, int idx_div,
+                          const int32_t* group_indices, int E, int64_t P, void* dst,
+                          int64_t ld_dst, int64_t features, int dtype, moe_stream_t stream);
 MOE_API int moe_k_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, const void* b,
                        int64_t b_rows, int64_t ldb, void* out,
                        const int32_t* group_indices, const void* indices, int idx_bytes,

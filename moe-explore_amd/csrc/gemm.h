@@ -60,5 +60,9 @@ bool m_grouped_mfma_dma_supported(const MGemmArgs& g);  // K % 64 == 0, 16-byte 
 int launch_m_grouped_mfma_dma(const MGemmArgs& g, hipStream_t stream);
 bool k_grouped_mfma_supported(const KGemmArgs& g);
 int launch_k_grouped_mfma(const KGemmArgs& g, hipStream_t stream);
+int launch_row_gather_kmajor(const void* src, int64_t src_rows, int64_t src_stride, const void* idx,
+                             int idx_bytes, int idx_div, const int32_t* group_indices, int E,
+                             int64_t P, void* dst, int64_t ld_dst, int64_t features, int dtype,
+                             hipStream_t stream);
 
 }  // namespace moe

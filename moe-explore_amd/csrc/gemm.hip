@@ -133,9 +133,12 @@ extern "C" int moe_k_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
   MOE_REQUIRE(dtype_bytes(dtype) != 0, "unknown dtype %d", dtype);
   MOE_REQUIRE(E >= 1 && Ka >= 0 && Nb >= 0 && topk >= 1, "bad sizes");
   MOE_REQUIRE(a_rows >= 0 && b_rows >= 0, "negative row count");
-  MOE_REQUIRE((flags & ~3) == 0, "unknown flag bits 0x%x", flags);
+  MOE_REQUIRE((flags & ~15) == 0, "unknown flag bits 0x%x", flags);
   const bool ga = flags & MOE_KGEMM_GATHER_A, gb = flags & MOE_KGEMM_GATHER_B;
+  const bool ka = flags & MOE_KGEMM_A_KMAJOR, kb = flags & MOE_KGEMM_B_KMAJOR;
   MOE_REQUIRE(!(ga && gb), "only one operand can be gathered");
+  MOE_REQUIRE(!(ka && kb) && !((ka || kb) && (ga || gb)),
+              "at most one operand is K-major, and then nothing is gathered");
   MOE_REQUIRE(group_indices != nullptr, "group_indices is null");
   if (ga || gb) {
     MOE_REQUIRE(indices != nullptr, "gather needs indices");
@@ -143,14 +146,52 @@ extern "C" int moe_k_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
   }
   if (Ka == 0 || Nb == 0) return MOE_OK;
   MOE_REQUIRE(out != nullptr, "out is null");
-  const int64_t P = ga ? b_rows : a_rows;
+  // (a K-major operand is [features, columns]: its "rows" argument counts columns)
+  const int64_t P = (ga || ka) ? b_rows : a_rows;
   MOE_REQUIRE(P <= 0x7fffffff, "too many rows");
   MOE_REQUIRE(P == 0 || (a != nullptr && b != nullptr && a_rows > 0 && b_rows > 0),
               "null or empty operand");
-  MOE_REQUIRE(lda >= Ka && ldb >= Nb, "row stride smaller than the row");
+  if (ka || kb) {
+    const int64_t need = moe_kmajor_columns(P, E);
+    MOE_REQUIRE((ka ? a_rows : b_rows) >= need && (ka ? lda : ldb) >= need,
+                "a K-major operand of %lld positions and %d experts has %lld columns",
+                (long long)P, E, (long long)need);
+    MOE_REQUIRE(ka ? ldb >= Nb : lda >= Ka, "row stride smaller than the row");
+  } else {
+    MOE_REQUIRE(lda >= Ka && ldb >= Nb, "row stride smaller than the row");
+  }
   KGemmArgs g{a, a_rows, lda, b, b_rows, ldb, out, group_indices, indices, idx_bytes,
               E, Ka,     Nb,  topk, flags, dtype, P, FastDiv(static_cast<uint32_t>(topk))};
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (!force_scalar() && k_grouped_mfma_supported(g)) return launch_k_grouped_mfma(g, s);
+  if (ka || kb)
+    return fail(MOE_ERR_UNSUPPORTED, "K-major operands need the MFMA kernel (16-bit dtype, widths and "
+                                     "strides multiples of 8, 16-byte aligned pointers)");
   return launch_k_grouped_generic(g, s);
+}
+
+extern "C" int64_t moe_kmajor_columns(int64_t P, int E) {
+  if (P < 0 || E < 1) return 0;
+  return 64 * (P / 64 + E + 1);
+}
+
+extern "C" int moe_row_gather_kmajor(const void* src, int64_t src_rows, int64_t src_stride,
+                                     const void* idx, int idx_bytes, int idx_div,
+                                     const int32_t* group_indices, int E, int64_t P, void* dst,
+                                     int64_t ld_dst, int64_t features, int dtype,
+                                     moe_stream_t stream) {
+  clear_error();
+  MOE_REQUIRE(dtype == MOE_DTYPE_BF16 || dtype == MOE_DTYPE_F16, "16-bit dtypes only, got %d", dtype);
+  MOE_REQUIRE(idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8, got %d", idx_bytes);
+  MOE_REQUIRE(idx_div >= 1 && E >= 1 && P >= 0 && P <= 0x7fffffff && features >= 0 && src_rows >= 0,
+              "bad sizes");
+  MOE_REQUIRE(group_indices != nullptr, "group_indices is null");
+  if (P == 0 || features == 0) return MOE_OK;
+  MOE_REQUIRE(src && idx && dst && src_rows > 0, "null or empty operand");
+  MOE_REQUIRE(ld_dst >= moe_kmajor_columns(P, E), "dst rows are shorter than moe_kmajor_columns(P, E)");
+  if (features % 8 != 0 || src_stride % 8 != 0 || ld_dst % 8 != 0 || !aligned16(src) || !aligned16(dst))
+    return fail(MOE_ERR_UNSUPPORTED, "row_gather_kmajor moves 16 bytes at a time: widths and strides "
+                                     "must be multiples of 8 elements, pointers 16-byte aligned");
+  return launch_row_gather_kmajor(src, src_rows, src_stride, idx, idx_bytes, idx_div, group_indices, E, P,
+                                  dst, ld_dst, features, dtype, static_cast<hipStream_t>(stream));
 }

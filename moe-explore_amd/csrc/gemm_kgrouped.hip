@@ -16,6 +16,14 @@
 // LDS so that every global store instruction writes whole 128-byte row pieces.
 // Experts without rows store zeros.  Workgroups are persistent (one per CU) and
 // run the K steps of all their tiles as one pipeline.
+//
+// K-major operand (MOE_KGEMM_A_KMAJOR / MOE_KGEMM_B_KMAJOR): the small operand of a weight
+// gradient is a set of gathered token rows that the caller has to materialise anyway.  Given
+// feature-major instead ([features, columns], the contraction index contiguous; written by
+// moe_row_gather_kmajor with every expert's segment starting on a multiple of 64 columns and
+// zero-filled up to the next one), its LDS tile is [256 features][64 positions] and its
+// fragments are plain 16-byte reads instead of two transpose loads each: with both operands
+// read through transpose loads the LDS, not the matrix cores, sets the pace of a K step.
 #include "gemm_mfma.h"
 
 #include <mutex>
@@ -174,15 +182,19 @@ constexpr int KLDS_BYTES = 5 * TILE_BYTES;   // 160 KiB, the whole LDS of a CU
 
 typedef const __attribute__((address_space(4))) int32_t* const_i32p;
 
-template <typename T, bool GA, bool GB>
+// KM: 0 = both operands position-major; 1 = a is K-major; 2 = b is K-major (then no gather).
+template <typename T, bool GA, bool GB, int KM>
 __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArgs g, KSched s,
                                                                         int ntiles) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr bool gathered = GA || GB;
+  static_assert(KM == 0 || !gathered, "a K-major operand is gathered by the caller");
   // The gathered operand (token rows: small, cache resident) is the SHORT one: two
   // LDS stages, copied one K step ahead.  The other operand streams from HBM: three
-  // stages, copied two steps ahead.  Without a gather, a is the short one.
-  constexpr bool A_SHORT = !GB;
+  // stages, copied two steps ahead.  Without a gather, a is the short one; a K-major
+  // operand always is.
+  constexpr bool A_SHORT = KM == 1 ? true : (KM == 2 ? false : !GB);
+  constexpr bool SKM = KM != 0;  // the short operand is K-major
   const int wpx = gridDim.x / kNumXcd;  // workgroups of an XCD = tiles of a chunk
   const int xcd = blockIdx.x % kNumXcd, within = blockIdx.x / kNumXcd;
   const int nch = (ntiles + wpx - 1) / wpx;
@@ -199,6 +211,7 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
 
   struct Tile {
     int e, mt, nt, lo, hi, KT;
+    int qs;  // first column of the expert's segment in a K-major operand
   };
   // round of this workgroup -> tile; false for the positions that pad the last chunk.  The
   // tiles of an expert are numbered block by block (blocks of GM x GN tiles, smaller ones at
@@ -236,6 +249,7 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
     t.lo = lo;
     t.hi = hi;
     t.KT = t.hi > t.lo ? (t.hi - t.lo + BK - 1) / BK : 0;
+    t.qs = 64 * ((lo >> 6) + t.e);
     return true;
   };
   auto store_zero_tile = [&](const Tile& t) {
@@ -259,6 +273,12 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
   const unsigned lds0 =
       __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<size_t>((lds_void*)smem))) +
       wave * 1024;
+  // K-major short operand: tile [256 features][64 positions], 128-byte rows; instruction i of
+  // wavefront w fills feature rows 64*i + 8*w .. +7 (lane -> row lane / 8, 16-byte chunk
+  // (lane & 7) ^ swizzle of the row, which is the same for all four instructions)
+  const int km_row = 8 * wave + (lane >> 3);
+  const int km_chunk = (lane & 7) ^ ((km_row >> 1) & 7);
+  int km_f0 = 0, km_last = 0;  // first feature row of the short cursor's tile, last row of the matrix
   const int64_t lda2 = g.lda * 2, ldb2 = g.ldb * 2;
   const int64_t ld_s2 = A_SHORT ? lda2 : ldb2, ld_l2 = A_SHORT ? ldb2 : lda2;
   const int s_last = static_cast<int>((A_SHORT ? g.a_rows : g.b_rows) - 1);
@@ -277,6 +297,12 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
   auto set_bases = [&](const Tile& t, bool is_a, const char*& plain) {
     const int64_t f0 = static_cast<int64_t>(is_a ? t.mt : t.nt) * (is_a ? KBM : KBN);
     const int64_t width = is_a ? g.Ka : g.Nb;
+    if (SKM && is_a == A_SHORT) {
+      km_f0 = static_cast<int>(f0);
+      km_last = static_cast<int>(width - 1);
+      plain = static_cast<const char*>(is_a ? g.a : g.b) + (static_cast<int64_t>(t.qs) + km_chunk * 8) * 2;
+      return;
+    }
     const bool gath = is_a ? GA : GB;
     const int64_t ld2 = is_a ? lda2 : ldb2;
     const char* base = static_cast<const char*>(is_a ? g.a : g.b);
@@ -329,6 +355,18 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
   auto issue_short = [&](int stage) {
     const unsigned base = lds0 + SHORT_BASE + stage * TILE_BYTES;
     const bool tail = cs.kt + 1 == cs.t.KT;
+    if constexpr (SKM) {
+      // (the columns past the end of the segment hold zeros: nothing to mask)
+      // (feature rows past the matrix only feed outputs that are not stored)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        int f = km_f0 + km_row + 64 * i;
+        f = f < km_last ? f : km_last;
+        copy16_to_lds(s_plain + f * ld_s2 + cs.kt * (BK * 2), base + i * 8192);
+      }
+      advance(cs, true);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const char* src;
@@ -374,16 +412,25 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
     s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(tile + nmajor16_off(k + 4, cbyte)));
     return __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
   };
+  auto read_km = [&](const char* tile, int kh, int row0) __attribute__((always_inline)) -> s16x8 {
+    return *reinterpret_cast<const s16x8*>(tile + kmajor_off(row0 + l16, kh * 4 + lg));
+  };
   auto read_unit_a = [&](int sstage, int lstage, int u, s16x8 (&af)[HB]) __attribute__((always_inline)) {
     const char* at = A_SHORT ? smem + SHORT_BASE + sstage * TILE_BYTES : smem + LONG_BASE + lstage * TILE_BYTES;
 #pragma unroll
-    for (int mb = 0; mb < HB; ++mb) af[mb] = read_tr(at, u >> 1, wm0 + ((u & 1) * HB + mb) * 16);
+    for (int mb = 0; mb < HB; ++mb) {
+      if constexpr (KM == 1) af[mb] = read_km(at, u >> 1, wm0 + ((u & 1) * HB + mb) * 16);
+      else af[mb] = read_tr(at, u >> 1, wm0 + ((u & 1) * HB + mb) * 16);
+    }
   };
   // b blocks [2*half, 2*half + 2) of K half kh
   auto read_unit_b = [&](int sstage, int lstage, int kh, int half, s16x8 (&bf)[NB16]) __attribute__((always_inline)) {
     const char* bt = A_SHORT ? smem + LONG_BASE + lstage * TILE_BYTES : smem + SHORT_BASE + sstage * TILE_BYTES;
 #pragma unroll
-    for (int nb = 2 * half; nb < 2 * half + 2; ++nb) bf[nb] = read_tr(bt, kh, wn0 + nb * 16);
+    for (int nb = 2 * half; nb < 2 * half + 2; ++nb) {
+      if constexpr (KM == 2) bf[nb] = read_km(bt, kh, wn0 + nb * 16);
+      else bf[nb] = read_tr(bt, kh, wn0 + nb * 16);
+    }
   };
   f32x4 acc[MB16][NB16];
   auto zero_acc = [&]() __attribute__((always_inline)) {
@@ -528,12 +575,67 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
   }
 }
 
+
+// Gathers token rows into the K-major operand layout of the weight-gradient kernel:
+//     dst[f, qs(e) + (p - lo(e))] = src[idx[p] / div, f]      p in [lo(e), hi(e))
+// with qs(e) = 64 * (lo(e) / 64 + e), and zeros from the end of the expert's segment up to the
+// next multiple of 64 columns.  A workgroup moves 64 positions x 64 features through LDS:
+// 128-byte row pieces in (gathered rows of src), 128-byte row pieces out (feature rows of dst).
+template <typename T>
+__global__ __launch_bounds__(256) void row_gather_kmajor_kernel(
+    const T* __restrict__ src, int64_t src_rows, int64_t src_stride, const void* __restrict__ idx,
+    int idx_bytes, FastDiv by_div, const int32_t* __restrict__ gi, int E, int P,
+    T* __restrict__ dst, int64_t ld_dst, int64_t features) {
+  __shared__ int sh[3];
+  __shared__ __attribute__((aligned(16))) T tile[64][64 + 8];
+  if (threadIdx.x < 64) find_tile<64>(gi, E, P, static_cast<int>(blockIdx.x), sh);
+  __syncthreads();
+  const int e = sh[0];
+  if (e < 0) return;
+  const int row0 = sh[1], end = sh[2];
+  int lo = gi[e];
+  lo = lo < 0 ? 0 : lo;
+  const int64_t col0 = 64 * static_cast<int64_t>((lo >> 6) + e) + (row0 - lo);
+  const int64_t f0 = static_cast<int64_t>(blockIdx.y) * 64;
+  const int t = threadIdx.x;
+  {  // in: position t / 4, features 16 * (t % 4) .. +15
+    const int pos = t >> 2;
+    const int p = row0 + pos;
+    int64_t srow = 0;
+    if (p < end) srow = clamp_index(by_div.div(load_index32(idx, idx_bytes, p)), src_rows);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int c = (t & 3) * 16 + h * 8;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (p < end && f0 + c < features)
+        v = *reinterpret_cast<const uint4*>(src + srow * src_stride + f0 + c);
+      *reinterpret_cast<uint4*>(&tile[pos][c]) = v;
+    }
+  }
+  __syncthreads();
+  {  // out: feature t / 4, positions 16 * (t % 4) .. +15
+    const int f = t >> 2;
+    if (f0 + f < features) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int q = (t & 3) * 16 + h * 8;
+        T v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = tile[q + j][f];
+        *reinterpret_cast<uint4*>(dst + (f0 + f) * ld_dst + col0 + q) = *reinterpret_cast<const uint4*>(v);
+      }
+    }
+  }
+}
+
 }  // namespace
 
 bool k_grouped_mfma_supported(const KGemmArgs& g) {
   if (g.dtype != MOE_DTYPE_BF16 && g.dtype != MOE_DTYPE_F16) return false;
   if (g.Ka % 8 != 0 || g.Nb % 8 != 0) return false;
   if (g.lda % 8 != 0 || g.ldb % 8 != 0) return false;
+  if ((g.flags & (MOE_KGEMM_A_KMAJOR | MOE_KGEMM_B_KMAJOR)) && (g.flags & (MOE_KGEMM_GATHER_A | MOE_KGEMM_GATHER_B)))
+    return false;
   if (!aligned16(g.a) || !aligned16(g.b) || !aligned16(g.out)) return false;
   if (g.P == 0) return false;  // nothing to contract: the scalar kernel writes the zeros
   return true;
@@ -588,17 +690,42 @@ int launch_k_grouped_mfma(const KGemmArgs& g, hipStream_t stream) {
     return MOE_OK;
   };
   const bool ga = g.flags & MOE_KGEMM_GATHER_A, gb = g.flags & MOE_KGEMM_GATHER_B;
+  const int km = (g.flags & MOE_KGEMM_A_KMAJOR) ? 1 : ((g.flags & MOE_KGEMM_B_KMAJOR) ? 2 : 0);
   int rc;
-  if (g.dtype == MOE_DTYPE_BF16)
-    rc = ga ? launch(k_grouped_persistent_kernel<bf16_t, true, false>)
-            : (gb ? launch(k_grouped_persistent_kernel<bf16_t, false, true>)
-                  : launch(k_grouped_persistent_kernel<bf16_t, false, false>));
-  else
-    rc = ga ? launch(k_grouped_persistent_kernel<f16_t, true, false>)
-            : (gb ? launch(k_grouped_persistent_kernel<f16_t, false, true>)
-                  : launch(k_grouped_persistent_kernel<f16_t, false, false>));
+  if (g.dtype == MOE_DTYPE_BF16) {
+    if (km == 1) rc = launch(k_grouped_persistent_kernel<bf16_t, false, false, 1>);
+    else if (km == 2) rc = launch(k_grouped_persistent_kernel<bf16_t, false, false, 2>);
+    else rc = ga ? launch(k_grouped_persistent_kernel<bf16_t, true, false, 0>)
+                 : (gb ? launch(k_grouped_persistent_kernel<bf16_t, false, true, 0>)
+                       : launch(k_grouped_persistent_kernel<bf16_t, false, false, 0>));
+  } else {
+    if (km == 1) rc = launch(k_grouped_persistent_kernel<f16_t, false, false, 1>);
+    else if (km == 2) rc = launch(k_grouped_persistent_kernel<f16_t, false, false, 2>);
+    else rc = ga ? launch(k_grouped_persistent_kernel<f16_t, true, false, 0>)
+                 : (gb ? launch(k_grouped_persistent_kernel<f16_t, false, true, 0>)
+                       : launch(k_grouped_persistent_kernel<f16_t, false, false, 0>));
+  }
   if (rc != MOE_OK) return rc;
   return check_launch("k_grouped_gemm (MFMA kernel)");
+}
+
+int launch_row_gather_kmajor(const void* src, int64_t src_rows, int64_t src_stride, const void* idx,
+                             int idx_bytes, int idx_div, const int32_t* group_indices, int E,
+                             int64_t P, void* dst, int64_t ld_dst, int64_t features, int dtype,
+                             hipStream_t stream) {
+  const int64_t blocks = P / 64 + E;  // static bound on the 64-position blocks of all experts
+  if (blocks > 0x7fffffff || (features + 63) / 64 > 65535) return fail(MOE_ERR_UNSUPPORTED, "grid too large");
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((features + 63) / 64));
+  const FastDiv by_div(static_cast<uint32_t>(idx_div));
+  if (dtype == MOE_DTYPE_BF16)
+    row_gather_kmajor_kernel<bf16_t><<<grid, 256, 0, stream>>>(
+        static_cast<const bf16_t*>(src), src_rows, src_stride, idx, idx_bytes, by_div, group_indices, E,
+        static_cast<int>(P), static_cast<bf16_t*>(dst), ld_dst, features);
+  else
+    row_gather_kmajor_kernel<f16_t><<<grid, 256, 0, stream>>>(
+        static_cast<const f16_t*>(src), src_rows, src_stride, idx, idx_bytes, by_div, group_indices, E,
+        static_cast<int>(P), static_cast<f16_t*>(dst), ld_dst, features);
+  return check_launch("row_gather_kmajor");
 }
 
 }  // namespace moe

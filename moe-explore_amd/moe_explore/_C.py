@@ -18,7 +18,7 @@ _lib = None
 DTYPE_F32, DTYPE_F16, DTYPE_BF16 = 0, 1, 2
 ACT_NONE, ACT_SILU, ACT_GELU, ACT_APPROX_GELU, ACT_SWIGLU, ACT_GEGLU = range(6)
 GEMM_GATHER_A, GEMM_SCATTER_C, GEMM_SCATTER_ADD, GEMM_SAVE_PREACT = 1, 2, 4, 8
-KGEMM_GATHER_A, KGEMM_GATHER_B = 1, 2
+KGEMM_GATHER_A, KGEMM_GATHER_B, KGEMM_A_KMAJOR, KGEMM_B_KMAJOR = 1, 2, 4, 8
 FP8_W_TILED = 4  # moe_m_grouped_gemm_fp8 only: weights stored tile-major
 ROUTER_SOFTMAX_FIRST, ROUTER_NORMALIZE, ROUTER_ERNIE = 1, 2, 4
 
@@ -51,6 +51,9 @@ SIGNATURES = {
                                   _vp, _vp, _i32, _vp, _i32, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i64, _vp]),
     "moe_k_grouped_gemm": (_i32, [_vp, _i64, _i64, _vp, _i64, _i64, _vp, _vp, _vp, _i32, _i32, _i64,
                                   _i64, _i32, _i32, _i32, _vp]),
+    "moe_kmajor_columns": (_i64, [_i64, _i32]),
+    "moe_row_gather_kmajor": (_i32, [_vp, _i64, _i64, _vp, _i32, _i32, _vp, _i32, _i64, _vp, _i64, _i64,
+                                     _i32, _vp]),
     "moe_act_bwd": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _i32, _vp, _i64, _vp, _i64,
                            _i64, _i32, _i32, _vp]),
     "moe_m_grouped_gemm_glu_bwd": (_i32, [_vp, _i64, _i64, _vp, _i64, _i64, _i64, _vp, _i64, _vp, _i64,

@@ -20,7 +20,7 @@ from moe_explore.functional.activation import activation, activation_name, is_gl
 from moe_explore.functional.scale_and_reduce import scale_and_reduce
 from moe_explore.router import router
 from moe_explore.expert_permute import get_token_indices
-from moe_explore.hip_kernels.row_gather_scatter import row_gather
+from moe_explore.hip_kernels.row_gather_scatter import row_gather, row_gather_kmajor
 from moe_explore.hip_kernels.m_grouped_gemm import (
     MGroupedGEMMParams,
     m_grouped_gemm,
@@ -167,14 +167,23 @@ class _ExpertsFunction(torch.autograd.Function):
             dh, a_scaled, dscale = act_bwd(h, g, act, row_scale=scores, permute_indices=idx,
                                            want_y_scaled=True, want_dscale=need_dscore)
         dw1 = dw2 = dx = dscores = None
-        # Weight gradients: the token rows are gathered first (one 20 us pass over R x d
-        # each).  The K-grouped kernel can gather by itself, but then has to wait for the
-        # row ids of every K step, and with them for the copies it keeps in flight:
-        # 10-15 % slower at this shape.
+        # Weight gradients: the token rows are gathered first, feature-major (one 25 us pass
+        # over R x d each): the K-grouped kernel then reads that operand from LDS with plain
+        # 16-byte loads instead of transpose loads (-10 % on dW1 at the Mixtral shape).  The
+        # kernel can also gather by itself, but then has to wait for the row ids of every K
+        # step, and with them for the copies it keeps in flight: 10-15 % slower.
         if ctx.needs_input_grad[2]:
-            dw2 = k_grouped_gemm(a_scaled, row_gather(dout, idx, topk), gi)
+            dt = row_gather_kmajor(dout, idx, topk, gi)
+            if dt is not None:
+                dw2 = k_grouped_gemm(a_scaled, dt, gi, b_kmajor=True)
+            else:
+                dw2 = k_grouped_gemm(a_scaled, row_gather(dout, idx, topk), gi)
         if ctx.needs_input_grad[1]:
-            dw1 = k_grouped_gemm(row_gather(x, idx, topk), dh, gi)
+            xt = row_gather_kmajor(x, idx, topk, gi)
+            if xt is not None:
+                dw1 = k_grouped_gemm(xt, dh, gi, a_kmajor=True)
+            else:
+                dw1 = k_grouped_gemm(row_gather(x, idx, topk), dh, gi)
         if ctx.needs_input_grad[0]:
             px = MGroupedGEMMParams(w1, gi, idx, False, True, T, topk, scales=None)
             ks = _ksplit_for(T * topk, w1.size(0), w1.size(1), w1.size(2))

@@ -183,13 +183,18 @@ def k_grouped_gemm(
     topk: int = 1,
     gather_a: bool = False,
     gather_b: bool = False,
+    a_kmajor: bool = False,
+    b_kmajor: bool = False,
 ):
     """Expert weight gradient: ``out[e] = a_e^T @ b_e`` with the contraction over
     expert ``e``'s sorted positions.  ``gather_a`` / ``gather_b`` read that operand's
-    row for position ``p`` at ``permute_indices[p] // topk``.  No reference
-    counterpart (the reference is forward-only)."""
+    row for position ``p`` at ``permute_indices[p] // topk``.  ``a_kmajor`` / ``b_kmajor``:
+    that operand is the feature-major matrix ``row_gather_kmajor`` returns (the fast path
+    for the gathered token rows).  No reference counterpart (the reference is
+    forward-only)."""
     assert a.dim() == 2 and b.dim() == 2 and a.dtype == b.dtype
-    assert not (gather_a and gather_b)
+    assert not (gather_a and gather_b) and not (a_kmajor and b_kmajor)
+    assert not ((a_kmajor or b_kmajor) and (gather_a or gather_b))
     _C.require_cuda(a, b, group_indices, permute_indices)
     if a.stride(1) != 1 and a.size(1) > 1:
         a = a.contiguous()
@@ -197,19 +202,24 @@ def k_grouped_gemm(
         b = b.contiguous()
     gi = _group_indices(group_indices)
     e = gi.numel() - 1
-    flags = (_C.KGEMM_GATHER_A if gather_a else 0) | (_C.KGEMM_GATHER_B if gather_b else 0)
+    flags = (_C.KGEMM_GATHER_A if gather_a else 0) | (_C.KGEMM_GATHER_B if gather_b else 0) | \
+        (_C.KGEMM_A_KMAJOR if a_kmajor else 0) | (_C.KGEMM_B_KMAJOR if b_kmajor else 0)
     perm = None
-    if flags:
+    if gather_a or gather_b:
         assert permute_indices is not None
         perm = permute_indices.contiguous()
         assert perm.numel() == (b.size(0) if gather_a else a.size(0))
-    else:
+    elif not (a_kmajor or b_kmajor):
         assert a.size(0) == b.size(0)
-    out = torch.empty((e, a.size(1), b.size(1)), device=a.device, dtype=a.dtype)
+    # a K-major operand is [features, columns]
+    ka = a.size(0) if a_kmajor else a.size(1)
+    nb = b.size(0) if b_kmajor else b.size(1)
+    out = torch.empty((e, ka, nb), device=a.device, dtype=a.dtype)
     st = _C.load().moe_k_grouped_gemm(
-        a.data_ptr(), a.size(0), a.stride(0), b.data_ptr(), b.size(0), b.stride(0), out.data_ptr(),
-        gi.data_ptr(), _C.ptr(perm), 0 if perm is None else _C.idx_bytes(perm), e, a.size(1),
-        b.size(1), topk, flags, _C.dtype_code(a.dtype), _C.stream_of(a))
+        a.data_ptr(), a.size(1) if a_kmajor else a.size(0), a.stride(0), b.data_ptr(),
+        b.size(1) if b_kmajor else b.size(0), b.stride(0), out.data_ptr(),
+        gi.data_ptr(), _C.ptr(perm), 0 if perm is None else _C.idx_bytes(perm), e, ka,
+        nb, topk, flags, _C.dtype_code(a.dtype), _C.stream_of(a))
     _C.check(st, "moe_k_grouped_gemm")
     return out
 

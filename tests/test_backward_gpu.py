@@ -110,6 +110,82 @@ def test_k_grouped_gemm_more_experts_than_the_balanced_deal_takes(E, Ka, Nb):
             assert_parity(out[e], ref[e], torch.bfloat16, f"expert {e} ({sizes[e]} rows)")
 
 
+@pytest.mark.parametrize("sizes,T,d,dtype", [
+    ([130, 0, 64, 1, 63, 65, 300, 0], 400, 72, torch.bfloat16),
+    ([1000, 1030, 990, 1076], 2048, 256, torch.bfloat16),
+    ([5] * 20, 77, 136, torch.float16),
+    ([0, 0, 700], 350, 64, torch.bfloat16),
+])
+def test_row_gather_kmajor_layout(sizes, T, d, dtype):
+    """moe_row_gather_kmajor: expert e's rows, transposed, start at column 64 * (lo // 64 + e)
+    and are followed by zeros up to the next multiple of 64 (exact: a copy)."""
+    from moe_explore.hip_kernels.row_gather_scatter import row_gather_kmajor
+    g = seeded(sum(sizes) + d)
+    E, R, k = len(sizes), sum(sizes), 2
+    gi = torch.zeros(E + 1, dtype=torch.int32)
+    gi[1:] = torch.cumsum(torch.tensor(sizes), 0)
+    slots = torch.randint(0, T * k, (R,), generator=g)
+    x = randn((T, d), g, dtype)
+    out = row_gather_kmajor(x.cuda(), slots.cuda(), k, gi.cuda())
+    assert out is not None and out.shape == (d, 64 * (R // 64 + E + 1))
+    out = out.cpu()
+    for e, n in enumerate(sizes):
+        lo = int(gi[e])
+        qs = 64 * (lo // 64 + e)
+        want = x[slots[lo:lo + n] // k].t()
+        assert torch.equal(out[:, qs:qs + n], want), f"expert {e}"
+        pad = (-n) % 64
+        if n:
+            assert (out[:, qs + n:qs + n + pad] == 0).all(), f"zero fill of expert {e}"
+
+
+@pytest.mark.parametrize("which", ["a", "b"])
+@pytest.mark.parametrize("sizes,Ka,Nb", [
+    ([700, 0, 515, 1300, 5, 600], 264, 520),
+    ([0, 1, 64, 65, 0, 130, 7, 0], 776, 2568),
+    ([1024, 1000, 1050, 1022], 512, 768),
+    ([max(0, int(2500 / (i + 1) ** 1.2) - 12) for i in range(64)], 256, 520),
+])
+def test_k_grouped_gemm_kmajor_operand(which, sizes, Ka, Nb):
+    """The weight-gradient GEMM with its gathered operand given feature-major
+    (row_gather_kmajor), against the oracle's gathered product."""
+    from moe_explore.hip_kernels.row_gather_scatter import row_gather_kmajor
+    from moe_explore.triton_kernels.m_grouped_gemm import k_grouped_gemm
+    g = seeded(sum(sizes) + Ka)
+    E, R, topk = len(sizes), sum(sizes), 2
+    T = (R + topk - 1) // topk
+    gi = torch.zeros(E + 1, dtype=torch.int32)
+    gi[1:] = torch.cumsum(torch.tensor(sizes), 0)
+    perm = torch.randperm(R, generator=g)
+    if which == "a":
+        a, b = randn((T, Ka), g, torch.bfloat16), randn((R, Nb), g, torch.bfloat16)
+        at = row_gather_kmajor(a.cuda(), perm.cuda(), topk, gi.cuda())
+        out = k_grouped_gemm(at, b.cuda(), gi.cuda(), a_kmajor=True)
+    else:
+        a, b = randn((R, Ka), g, torch.bfloat16), randn((T, Nb), g, torch.bfloat16)
+        bt = row_gather_kmajor(b.cuda(), perm.cuda(), topk, gi.cuda())
+        out = k_grouped_gemm(a.cuda(), bt, gi.cuda(), b_kmajor=True)
+    ref = moe_ref.k_grouped_matmul(a, b, gi, perm, topk, which == "a", which == "b")
+    assert out.shape == (E, Ka, Nb)
+    assert_parity(out, ref, torch.bfloat16, f"k_grouped_gemm, K-major {which}")
+    for e, n in enumerate(sizes):
+        if n == 0:
+            assert (out[e] == 0).all()
+        elif e % 9 == 0 or n < 8:
+            assert_parity(out[e], ref[e], torch.bfloat16, f"expert {e} ({n} rows)")
+
+
+def test_k_grouped_gemm_kmajor_is_refused_outside_the_mfma_kernel():
+    from moe_explore import _C
+    from moe_explore.hip_kernels.row_gather_scatter import row_gather_kmajor
+    g = seeded(3)
+    x = randn((40, 36), g, torch.float32)
+    gi = torch.tensor([0, 30, 64], dtype=torch.int32)
+    assert row_gather_kmajor(x.cuda(), torch.arange(64).cuda(), 2, gi.cuda()) is None   # fp32
+    xb = randn((40, 36), g, torch.bfloat16)                                              # 36 % 8 != 0
+    assert row_gather_kmajor(xb.cuda(), torch.arange(64).cuda(), 2, gi.cuda()) is None
+
+
 @pytest.mark.parametrize("which", ["a", "b"])
 def test_k_grouped_gemm_gather(which):
     from moe_explore.expert_permute import get_token_indices
