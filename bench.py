@@ -125,7 +125,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--mode", choices=["fwdbwd", "fwd"], default="fwdbwd")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23", "fp8", "digest"],
+    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23", "fp8", "digest", "ablation"],
                     default="all",
                     help="profiling aids: 'kernel' launches only the dominant GEMM --steps times, "
                          "'copy' only a 1 GiB device copy (the known-size kernel that calibrates "
@@ -137,8 +137,11 @@ def main():
                          "backward) at the shapes of configs 2 and 3, config 3 with Zipf(1.2) expert "
                          "loads, 'fp8' the fp8 inference layer (config 4: T = 128, 1024, 8192, GeGLU) "
                          "with its weight-streaming rate and TFLOP/s, 'digest' prints the digest of "
-                         "the dominant kernel's sources that a profile summary records; none of "
-                         "them prints the JSON line")
+                         "the dominant kernel's sources that a profile summary records, 'ablation' times "
+                         "the four GEMM shapes of config 1 (gate/up, dX, G without its fused epilogue, "
+                         "dW1 and dW2) with evenly loaded experts on N(0,1) and on all-zero operands, "
+                         "for runs with MOE_HIP_LIB pointing at a `build.py --ablate N` library; none "
+                         "of them prints the JSON line")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path; run with --gpus 1",
@@ -166,6 +169,51 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print("copied 1 GiB x %d" % args.steps)
+        return
+    if args.only == "ablation":
+        from moe_explore.hip_kernels.row_gather_scatter import row_gather_kmajor
+        from moe_explore.testing import perfect_routing
+        from moe_explore.triton_kernels.m_grouped_gemm import k_grouped_gemm
+        T, d, ff, E, k = cfg["T"], cfg["d"], cfg["ff"], cfg["E"], cfg["k"]
+        R = T * k
+        tag = os.path.basename(_C.lib_path())
+
+        def timed(fn, flops, what, kind):
+            for _ in range(args.warmup):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                fn()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) / args.steps * 1e3
+            print("%-28s %-5s %-46s %7.3f ms %7.1f TFLOP/s" % (tag, kind, what, ms, flops / ms / 1e9), flush=True)
+
+        for kind in ("rand", "zero"):
+            torch.manual_seed(0)
+            mk = (lambda *s: torch.randn(*s, device=dev, dtype=torch.bfloat16)) if kind == "rand" else \
+                (lambda *s: torch.zeros(*s, device=dev, dtype=torch.bfloat16))
+            w1, w2 = mk(E, d, 2 * ff) * 0.02, mk(E, ff, d) * 0.02
+            x, dout, dh, a = mk(T, d), mk(T, d), mk(R, 2 * ff), mk(R, ff)
+            _, idx = perfect_routing(T, E, k, dev, torch.bfloat16)
+            p = get_token_indices(idx.view(T, k), k, E, zero_prefix=True)
+            out = torch.empty((R, ff), device=dev, dtype=torch.bfloat16)
+            gu = MGroupedGEMMParams(w1, p.group_indices, p.indices, True, False, T, k, activation="swiglu")
+            px = MGroupedGEMMParams(w1, p.group_indices, p.indices, False, True, T, k)
+            pg = MGroupedGEMMParams(w2, p.group_indices, p.indices, True, False, T, k)
+            xt = row_gather_kmajor(x, p.indices, k, p.group_indices)
+            dt = row_gather_kmajor(dout, p.indices, k, p.group_indices)
+            with torch.no_grad():
+                timed(lambda: m_grouped_gemm(x, gu, out=out), 4.0 * R * d * ff, "gate/up (N-contiguous W, gather, swiglu)", kind)
+                timed(lambda: m_grouped_gemm(dh, px, transpose_weight=True), 4.0 * R * d * ff,
+                      "dX (K-contiguous W, K = 2 ff, scatter)", kind)
+                timed(lambda: m_grouped_gemm(dout, pg, transpose_weight=True), 2.0 * R * d * ff,
+                      "G (K-contiguous W, K = d, gather, no epilogue)", kind)
+                timed(lambda: k_grouped_gemm(xt, dh, p.group_indices, a_kmajor=True), 4.0 * R * d * ff,
+                      "dW1 (K-grouped, a K-major)", kind)
+                timed(lambda: k_grouped_gemm(a, dt, p.group_indices, b_kmajor=True), 2.0 * R * d * ff,
+                      "dW2 (K-grouped, b K-major)", kind)
+            del w1, w2, x, dout, dh, a, out, xt, dt
         return
     if args.only == "fp8":
         from moe_explore.fp8 import Fp8MLPParams, quantize_expert_weights, routed_experts_fp8

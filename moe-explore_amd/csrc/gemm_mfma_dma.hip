@@ -31,6 +31,16 @@
 
 #include <stdlib.h>
 
+// Ablation builds (`build.py --ablate N`; never the product library): parts of the K loop
+// are left out, the results are wrong and only the run time is of interest.  It answers what a
+// K step spends on what: bit 1 skips half of the token-fragment LDS reads, 8 all of them, 4
+// the weight-fragment reads, 2 the global -> LDS copies of the loop, 16 / 32 make the token /
+// weight copies cycle through eight K steps (an L2-resident window: same LDS traffic, no
+// fabric or HBM traffic).  0 compiles to the product kernel, instruction for instruction.
+#ifndef MOE_ABLATE
+#define MOE_ABLATE 0
+#endif
+
 #include <mutex>
 #include <unordered_map>
 
@@ -198,14 +208,16 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
 #pragma unroll
     for (int i = 0; i < A_INSTR; ++i)
       if (i >= first && i < last && 8 * (NWAVES * i + wave) < rows_here)
-        copy16_to_lds(g.a, a_src[i] + static_cast<uint32_t>(kt0 + kt) * (BK * 2), base + i * (NWAVES * 1024));
+        copy16_to_lds(g.a, a_src[i] + static_cast<uint32_t>((MOE_ABLATE & 16) ? ((kt0 + kt) & 7) : (kt0 + kt)) * (BK * 2),
+                      base + i * (NWAVES * 1024));
   };
   auto issue_weight_copies = [&](int wstage, int kt, int first, int last) __attribute__((always_inline)) {
     const unsigned base = lds0 + W_BASE + wstage * W_BYTES;
 #pragma unroll
     for (int i = 0; i < W_INSTR; ++i)
       if (i >= first && i < last)
-        copy16_to_lds(wbase, w_src[i] + static_cast<uint32_t>(kt0 + kt) * w_step, base + i * (NWAVES * 1024));
+        copy16_to_lds(wbase, w_src[i] + static_cast<uint32_t>((MOE_ABLATE & 32) ? ((kt0 + kt) & 7) : (kt0 + kt)) * w_step,
+                      base + i * (NWAVES * 1024));
   };
 
   // ---- LDS -> fragment addresses --------------------------------------------------
@@ -350,30 +362,30 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
       const int wahead = wnext == 2 ? 0 : wnext + 1;
       const bool more = gs + 1 < S, ahead = gs + 2 < S;
       const bool tile_ends = kt + 1 == KT;
-      if (more) issue_token_copies(stage ^ 1, kt_a, 0, AH);
+      if (more && !(MOE_ABLATE & 2)) issue_token_copies(stage ^ 1, kt_a, 0, AH);
       __builtin_amdgcn_s_setprio(2);
       __builtin_amdgcn_sched_barrier(0);
-      read_unit_w(wcur, 0, 1, wfP, blocks);
-      read_unit_t(stage, 1, tfB, blocks);
+      if (!(MOE_ABLATE & 4)) read_unit_w(wcur, 0, 1, wfP, blocks);
+      if (!(MOE_ABLATE & 9)) read_unit_t(stage, 1, tfB, blocks);
       multiply_unit(0, tfA, wfP, blocks);
       interleave_unit();
       if (more) {
-        issue_token_copies(stage ^ 1, kt_a, AH, A_INSTR);
+        if (!(MOE_ABLATE & 2)) issue_token_copies(stage ^ 1, kt_a, AH, A_INSTR);
         advance_a();
       }
       __builtin_amdgcn_sched_barrier(0);
-      read_unit_w(wcur, 1, 0, wfQ, blocks);
-      read_unit_t(stage, 2, tfA, blocks);
+      if (!(MOE_ABLATE & 4)) read_unit_w(wcur, 1, 0, wfQ, blocks);
+      if (!(MOE_ABLATE & 8)) read_unit_t(stage, 2, tfA, blocks);
       multiply_unit(1, tfB, wfP, blocks);
       interleave_unit();
-      if (ahead) issue_weight_copies(wahead, kt_w, 0, WH);
+      if (ahead && !(MOE_ABLATE & 2)) issue_weight_copies(wahead, kt_w, 0, WH);
       __builtin_amdgcn_sched_barrier(0);
-      read_unit_w(wcur, 1, 1, wfQ, blocks);
-      read_unit_t(stage, 3, tfB, blocks);
+      if (!(MOE_ABLATE & 4)) read_unit_w(wcur, 1, 1, wfQ, blocks);
+      if (!(MOE_ABLATE & 9)) read_unit_t(stage, 3, tfB, blocks);
       multiply_unit(0, tfA, wfQ, blocks);
       interleave_unit();
       if (ahead) {
-        issue_weight_copies(wahead, kt_w, WH, W_INSTR);
+        if (!(MOE_ABLATE & 2)) issue_weight_copies(wahead, kt_w, WH, W_INSTR);
         advance_w();
       }
       __builtin_amdgcn_s_setprio(0);
@@ -385,8 +397,8 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
         // (the first fragments of a next tile are read after the store of this one:
         // held across the store they would crowd the register file)
         if (!tile_ends) {
-          read_unit_t(stage ^ 1, 0, tfA, blocks);
-          read_unit_w(wnext, 0, 0, wfP, blocks);
+          if (!(MOE_ABLATE & 8)) read_unit_t(stage ^ 1, 0, tfA, blocks);
+          if (!(MOE_ABLATE & 4)) read_unit_w(wnext, 0, 0, wfP, blocks);
         }
       }
       multiply_unit(1, tfB, wfQ, blocks);
