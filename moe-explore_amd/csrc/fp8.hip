@@ -325,26 +325,34 @@ __global__ __launch_bounds__(kThreads) void m_grouped_fp8_kernel(Fp8Args fa, Sch
 
   // ---- dequantise: acc * a_scale[row] * w_scale[e, n] -----------------------------------
   const float* wsc = fa.w_scale + static_cast<int64_t>(expert) * g.N;
+  float as[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     int p = row0 + wm0 + mb * 32 + l32;
     p = p < end ? p : end - 1;
     int64_t arow = p;
     if (g.flags & MOE_GEMM_GATHER_A) arow = g.by_topk.div(load_index32(g.indices, g.idx_bytes, p));
-    const float as = fa.a_scale[clamp_index(arow, g.a_rows)];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int run = 0; run < 4; ++run) {
-        int64_t n = n0 + wn0 + nb * 32 + run * 8 + lhi * 4;
-        n = n + 3 < g.N ? n : g.N - 4;  // N is a multiple of 8; columns past N are not stored
-        const float4 ws = *reinterpret_cast<const float4*>(wsc + n);
-        acc[mb][nb][run * 4 + 0] *= as * ws.x;
-        acc[mb][nb][run * 4 + 1] *= as * ws.y;
-        acc[mb][nb][run * 4 + 2] *= as * ws.z;
-        acc[mb][nb][run * 4 + 3] *= as * ws.w;
-      }
+    as[mb] = fa.a_scale[clamp_index(arow, g.a_rows)];
   }
+  // One run of four channel scales at a time (and a scheduling barrier after it): with all
+  // eight float4 loads hoisted next to the 128 accumulators the 256-row kernel spilled 31-40
+  // registers a lane to scratch, 80 KiB written and read back per tile.
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+    for (int run = 0; run < 4; ++run) {
+      int64_t n = n0 + wn0 + nb * 32 + run * 8 + lhi * 4;
+      n = n + 3 < g.N ? n : g.N - 4;  // N is a multiple of 8; columns past N are not stored
+      const float4 ws = *reinterpret_cast<const float4*>(wsc + n);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        acc[mb][nb][run * 4 + 0] *= as[mb] * ws.x;
+        acc[mb][nb][run * 4 + 1] *= as[mb] * ws.y;
+        acc[mb][nb][run * 4 + 2] *= as[mb] * ws.z;
+        acc[mb][nb][run * 4 + 3] *= as[mb] * ws.w;
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
 
   if (lds_epilogue_ok<T>(g)) {
     __syncthreads();
