@@ -127,10 +127,11 @@ struct Fp8Args {
   int w_tiled;  // weights stored as the LDS images of their (column tile, K step) blocks
 };
 
-__device__ __forceinline__ void copy16_to_lds(const void* src, unsigned lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+// One 1 KiB copy instruction: lane i's 16 bytes at base + offset go to LDS address M0 + 16 i.
+__device__ __forceinline__ void copy16_to_lds(const void* base, uint32_t offset, unsigned lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(lds_addr), "v"(src)
+               : "s"(lds_addr), "v"(offset), "s"(base)
                : "memory");
 }
 __device__ __forceinline__ void wait_copies_and_barrier() {
@@ -143,12 +144,31 @@ __device__ __forceinline__ void wait_copies_keep_youngest_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(YOUNGEST) : "memory");
 }
 
+struct NextDraw {
+  unsigned* slot;   // queue word the next draw goes to (nullptr: every queue has run dry)
+  unsigned value;   // what the draw returned (thread 0)
+  bool drawn;
+};
+
+// One work item: `tpw` adjacent column tiles of one row block, computed as ONE stream of K
+// steps (token addresses stay, weight addresses move on), so that the copies of the next
+// tile's first steps fly while the finished accumulators are stored.  A gate/up tile of
+// config 4 has only 32 K steps: what a work item pays once (tile lookup, index fetch, the
+// latency of the first copies, the store) weighs twice what it does in the 16-bit kernel.
+// 2 x 4 wavefronts, a wavefront tile of BM/2 x 64 = MB x 2 blocks of 32 x 32; a K step of 128
+// is four units (K half x token-row half) of MB MFMAs; the fragments of the next unit are read
+// while a unit is multiplied, and the weight fragments of a K half serve both of its units.
 template <typename T, int BM, int ACT>
-__global__ __launch_bounds__(kThreads) void m_grouped_fp8_kernel(Fp8Args fa, Sched s) {
+__device__ __forceinline__ void fp8_work_item(const Fp8Args& fa, const Sched s, const int id,
+                                              NextDraw& next) {
   MGemmArgs g = fa.g;
+  constexpr int NWAVES = WAVES_M * WAVES_N;
   constexpr int WM = BM / WAVES_M;
-  constexpr int MB = WM / 32;
-  constexpr int A_INSTR = BM / 64, W_INSTR = BN / 64;
+  constexpr int MB = WM / 32;   // 32-row blocks of a wavefront
+  constexpr int HB = MB / 2;    // token blocks of one unit
+  static_assert(NWAVES == 8 && NB == 2 && HB >= 1, "2 x 4 wavefronts of BM/2 x 64");
+  constexpr int A_INSTR = BM / 8 / NWAVES;  // 1 KiB copy instructions per wavefront, token tile
+  constexpr int W_INSTR = 32 / NWAVES;
   constexpr int A_BYTES = BM * 128, W_BYTES = BN * 128;
   // LDS: two token stages, then three weight stages.  Weights are copied two K steps
   // ahead, tokens one: with few rows per expert the kernel only streams weights, and
@@ -163,226 +183,455 @@ __global__ __launch_bounds__(kThreads) void m_grouped_fp8_kernel(Fp8Args fa, Sch
   int mt, nt;
   {
     const int ch = s.GM * s.GN;
-    const int id = blockIdx.x;
     const int xcd = id % kNumXcd, j = id / kNumXcd;
-    const int blk = (j / ch) * kNumXcd + xcd, within = j % ch;
-    const int blk_m = blk / s.nblk_n, blk_n = blk - blk_m * s.nblk_n;
-    mt = blk_m * s.GM + within % s.GM;
-    nt = blk_n * s.GN + within / s.GM;
+    const int jb = s.by_block.div(j);
+    const int blk = jb * kNumXcd + xcd, within = j - jb * ch;
+    const int blk_m = s.by_nblk_n.div(blk), blk_n = blk - blk_m * s.nblk_n;
+    const int wq = s.by_gm.div(within);
+    mt = blk_m * s.GM + (within - wq * s.GM);
+    nt = blk_n * s.GN + wq;
     if (nt >= s.NT) return;
   }
   // a K part of a tile is scheduled like a column tile of its own
-  const int real_nt = s.NT / s.ksplit;
-  const int kpart = nt / real_nt;
-  nt -= kpart * real_nt;
+  const int kpart = s.by_real_nt.div(nt);
+  nt -= kpart * s.real_nt;
   const int KT = static_cast<int>(g.K / BKQ) / s.ksplit;  // K steps of this part
-  const int64_t kt0 = static_cast<int64_t>(kpart) * KT;
+  const int kt0 = kpart * KT;
   g.c = static_cast<char*>(g.c) + static_cast<int64_t>(kpart) * g.c_split_stride * sizeof(T);
   if (threadIdx.x < 64) find_tile<BM>(g.group_indices, g.E, static_cast<int>(g.P), mt, sh_tile);
   __syncthreads();
-  const int expert = sh_tile[0];
+  const int expert = __builtin_amdgcn_readfirstlane(sh_tile[0]);
   if (expert < 0) return;
   const int row0 = sh_tile[1], end = sh_tile[2];
-  const int64_t n0 = static_cast<int64_t>(nt) * BN;
+  // column tiles nt0 .. nt0 + ntiles - 1 of this row block
+  const int nt0 = nt * s.tpw;
+  const int col_tiles = static_cast<int>((g.N + BN - 1) / BN);
+  const int ntiles = col_tiles - nt0 < s.tpw ? col_tiles - nt0 : s.tpw;
 
-  const int tid = threadIdx.x, lane = tid & 63;
+  // (opaque: what depends only on the thread id would otherwise be computed once for all the
+  // work items of the workgroup and held in registers across them, next to the accumulators)
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm0 = (wave / WAVES_N) * WM, wn0 = (wave % WAVES_N) * WN;
   const int l32 = lane & 31, lhi = lane >> 5;
 
-  const char* a_src[A_INSTR];
+  // ---- global source of every copy instruction: a wave-uniform base + 32-bit byte offset ----
+  // token tile: instruction i of wavefront w fills rows 8*(8i + w) .. +7, lane -> (row, chunk).
+  // Rows that are not gathered are addressed from the first row of the block, so only a
+  // gathered token matrix has to stay below 4 GiB (checked on the host).
+  const bool gather = g.flags & MOE_GEMM_GATHER_A;
+  const char* const abase = static_cast<const char*>(g.a) + (gather ? 0 : static_cast<int64_t>(row0) * g.lda);
+  uint32_t a_src[A_INSTR];
+  float a_scale[MB];  // activation scale of this lane's row in every row block of the wavefront
 #pragma unroll
   for (int i = 0; i < A_INSTR; ++i) {
-    const int r = 8 * (8 * i + wave) + (lane >> 3);
+    const int r = 8 * (NWAVES * i + wave) + (lane >> 3);
     const int c = (lane & 7) ^ ((r >> 1) & 7);
     int p = row0 + r;
     p = p < end ? p : end - 1;
     int64_t arow = p;
-    if (g.flags & MOE_GEMM_GATHER_A) arow = g.by_topk.div(load_index32(g.indices, g.idx_bytes, p));
+    if (gather) arow = g.by_topk.div(load_index32(g.indices, g.idx_bytes, p));
     arow = clamp_index(arow, g.a_rows);
-    a_src[i] = static_cast<const char*>(g.a) + arow * g.lda + c * 16 + kt0 * BKQ;
+    a_src[i] = static_cast<uint32_t>((arow - (gather ? 0 : row0)) * g.lda + c * 16);
   }
-  const char* w_src[W_INSTR];
-  int64_t w_kstep;  // bytes from one K step to the next
-  if (fa.w_tiled) {
-    // tile-major weights: the 32 KiB of column tile nt, K step kt are stored contiguously,
-    // in the order (and with the swizzle) of the LDS tile, so a step is one linear copy
-    // and the whole tile one sequential stream
-    const int64_t tile = static_cast<int64_t>(expert) * real_nt + nt;
-    const char* wbase = static_cast<const char*>(g.w) + (tile * (g.K / BKQ) + kt0) * W_BYTES;
-#pragma unroll
-    for (int i = 0; i < W_INSTR; ++i) w_src[i] = wbase + (8 * i + wave) * 1024 + lane * 16;
-    w_kstep = W_BYTES;
-  } else {
-    const char* wbase = static_cast<const char*>(g.w) + static_cast<int64_t>(expert) * g.ldw_e;
-#pragma unroll
-    for (int i = 0; i < W_INSTR; ++i) {
-      const int r = 8 * (8 * i + wave) + (lane >> 3);
-      const int c = (lane & 7) ^ ((r >> 1) & 7);
-      int64_t n = n0 + r;
-      n = n < g.N ? n : g.N - 1;
-      w_src[i] = wbase + n * g.ldw_n + c * 16 + kt0 * BKQ;
-    }
-    w_kstep = BKQ;
-  }
-  const unsigned lds0 =
-      __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<size_t>((lds_void*)smem))) +
-      wave * 1024;
-  auto issue_token_copies = [&](int stage, int kt) {
-    const unsigned base = lds0 + stage * A_BYTES;
-#pragma unroll
-    for (int i = 0; i < A_INSTR; ++i)
-      copy16_to_lds(a_src[i] + static_cast<int64_t>(kt) * BKQ, base + i * 8192);
-  };
-  auto issue_weight_copies = [&](int wstage, int kt) {
-    const unsigned base = lds0 + W_BASE + wstage * W_BYTES;
-#pragma unroll
-    for (int i = 0; i < W_INSTR; ++i)
-      copy16_to_lds(w_src[i] + kt * w_kstep, base + i * 8192);
-  };
-
-  // a lane's fragment of a 32-row block for sub-step kk: 32 bytes = chunks 4kk + 2lhi, +1
-  auto read32 = [&](const char* tile, int row, int kk) -> i32x8 {
-    const i32x4 lo = *reinterpret_cast<const i32x4*>(tile + kmajor_off(row, kk * 4 + lhi * 2));
-    const i32x4 hi = *reinterpret_cast<const i32x4*>(tile + kmajor_off(row, kk * 4 + lhi * 2 + 1));
-    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-  };
-  f32x16 acc[MB][NB];
-#pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.0f;
-
-  // Fragments are 32 bytes per lane and block, so a full second set would not fit
-  // in the register file next to the accumulators.  The token fragments roll: once
-  // the MFMAs of row block mb are issued, its registers take the fragment of the
-  // next sub-step; only the weight fragments (used by every row block) are kept
-  // twice.  `next` = false on the very last sub-step.
-  i32x8 tf[MB], wfa[NB], wfb[NB];
-  auto substep = [&](i32x8 (&wf_cur)[NB], i32x8 (&wf_next)[NB], int next_stage, int next_wstage,
-                     int next_kk, auto next_tag) {
-    constexpr bool next = decltype(next_tag)::value;
-    const char* at = smem + next_stage * A_BYTES;
-    const char* wt = smem + W_BASE + next_wstage * W_BYTES;
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        acc[mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-            wf_cur[nb], tf[mb], acc[mb][nb], 0 /* A: e4m3 */, 0 /* B: e4m3 */, 0, 127, 0, 127);
-      if constexpr (next) {
-        if (mb < NB) wf_next[mb] = read32(wt, wn0 + mb * 32 + l32, next_kk);
-        tf[mb] = read32(at, wm0 + mb * 32 + l32, next_kk);
-      }
-    }
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      __builtin_amdgcn_sched_group_barrier(0x008, NB, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-
-  issue_token_copies(0, 0);
-  issue_weight_copies(0, 0);
-  if (KT > 1) {
-    issue_weight_copies(1, 1);
-    wait_copies_keep_youngest_and_barrier<W_INSTR>();
-  } else {
-    wait_copies_and_barrier();
-  }
-  {
-    const char* at = smem;
-    const char* wt = smem + W_BASE;
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) wfa[nb] = read32(wt, wn0 + nb * 32 + l32, 0);
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) tf[mb] = read32(at, wm0 + mb * 32 + l32, 0);
-  }
-  using yes = std::integral_constant<bool, true>;
-  using no = std::integral_constant<bool, false>;
-  int wcur = 0;  // weight stage of step kt: kt % 3
-  for (int kt = 0; kt < KT - 1; ++kt) {
-    const int stage = kt & 1;
-    const int wnext = wcur == 2 ? 0 : wcur + 1;
-    const int wahead = wnext == 2 ? 0 : wnext + 1;
-    const bool ahead = kt + 2 < KT;
-    issue_token_copies(stage ^ 1, kt + 1);
-    __builtin_amdgcn_sched_barrier(0);
-    substep(wfa, wfb, stage, wcur, 1, yes{});
-    if (ahead) issue_weight_copies(wahead, kt + 2);
-    // the token copies of step kt+1 and the weight copies of step kt+1 (issued a step
-    // earlier) must have landed; the weight copies of step kt+2 may still fly
-    if (ahead) wait_copies_keep_youngest_and_barrier<W_INSTR>();
-    else wait_copies_and_barrier();
-    substep(wfb, wfa, stage ^ 1, wnext, 0, yes{});
-    wcur = wnext;
-  }
-  substep(wfa, wfb, (KT - 1) & 1, wcur, 1, yes{});
-  substep(wfb, wfa, 0, 0, 0, no{});
-
-  // ---- dequantise: acc * a_scale[row] * w_scale[e, n] -----------------------------------
-  const float* wsc = fa.w_scale + static_cast<int64_t>(expert) * g.N;
-  float as[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     int p = row0 + wm0 + mb * 32 + l32;
     p = p < end ? p : end - 1;
     int64_t arow = p;
-    if (g.flags & MOE_GEMM_GATHER_A) arow = g.by_topk.div(load_index32(g.indices, g.idx_bytes, p));
-    as[mb] = fa.a_scale[clamp_index(arow, g.a_rows)];
+    if (gather) arow = g.by_topk.div(load_index32(g.indices, g.idx_bytes, p));
+    a_scale[mb] = fa.a_scale[clamp_index(arow, g.a_rows)];
   }
-  // One run of four channel scales at a time (and a scheduling barrier after it): with all
-  // eight float4 loads hoisted next to the 128 accumulators the 256-row kernel spilled 31-40
-  // registers a lane to scratch, 80 KiB written and read back per tile.
+  uint32_t w_src[W_INSTR];
+  const char* wbase;  // weights of this expert (tile-major: of its current column tile)
+  uint32_t w_step;    // bytes from one K step to the next
+  auto set_w_src = [&](int tile) __attribute__((always_inline)) {  // weight sources of column tile nt0 + tile
+    if (fa.w_tiled) {
+      // tile-major weights: the 32 KiB of a column tile and K step are stored contiguously,
+      // in the order (and with the swizzle) of the LDS tile, so a step is one linear copy
+      // and the whole tile one sequential stream
+      const int64_t t = static_cast<int64_t>(expert) * col_tiles + nt0 + tile;
+      wbase = static_cast<const char*>(g.w) + t * (g.K / BKQ) * W_BYTES;
+    } else {
+      const int64_t n0 = static_cast<int64_t>(nt0 + tile) * BN;
 #pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
+      for (int i = 0; i < W_INSTR; ++i) {
+        const int r = 8 * (NWAVES * i + wave) + (lane >> 3);
+        const int c = (lane & 7) ^ ((r >> 1) & 7);
+        int64_t n = n0 + r;
+        n = n < g.N ? n : g.N - 1;
+        w_src[i] = static_cast<uint32_t>(n * g.ldw_n + c * 16);
+      }
+    }
+  };
+  if (fa.w_tiled) {
 #pragma unroll
-    for (int run = 0; run < 4; ++run) {
-      int64_t n = n0 + wn0 + nb * 32 + run * 8 + lhi * 4;
-      n = n + 3 < g.N ? n : g.N - 4;  // N is a multiple of 8; columns past N are not stored
-      const float4 ws = *reinterpret_cast<const float4*>(wsc + n);
+    for (int i = 0; i < W_INSTR; ++i) w_src[i] = (NWAVES * i + wave) * 1024 + lane * 16;
+    w_step = W_BYTES;
+  } else {
+    wbase = static_cast<const char*>(g.w) + static_cast<int64_t>(expert) * g.ldw_e;
+    w_step = BKQ;
+  }
+  set_w_src(0);
+  const unsigned lds0 =
+      __builtin_amdgcn_readfirstlane(static_cast<unsigned>(reinterpret_cast<size_t>((lds_void*)smem))) +
+      wave * 1024;
+
+  // Copy instructions [first, last) of a tile; the main loop spreads them over the units of a
+  // K step so that they do not queue up in front of the MFMAs.  A copy instruction whose eight
+  // token rows all lie past the end of the group is not issued: those LDS rows keep stale data
+  // and only feed rows that are never stored.
+  const int rows_here = __builtin_amdgcn_readfirstlane(end - row0);
+  auto issue_token_copies = [&](int stage, int kt, int first, int last) __attribute__((always_inline)) {
+    const unsigned base = lds0 + stage * A_BYTES;
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        acc[mb][nb][run * 4 + 0] *= as[mb] * ws.x;
-        acc[mb][nb][run * 4 + 1] *= as[mb] * ws.y;
-        acc[mb][nb][run * 4 + 2] *= as[mb] * ws.z;
-        acc[mb][nb][run * 4 + 3] *= as[mb] * ws.w;
+    for (int i = 0; i < A_INSTR; ++i)
+      if (i >= first && i < last && 8 * (NWAVES * i + wave) < rows_here)
+        copy16_to_lds(abase, a_src[i] + static_cast<uint32_t>(kt0 + kt) * BKQ, base + i * (NWAVES * 1024));
+  };
+  auto issue_weight_copies = [&](int wstage, int kt, int first, int last) __attribute__((always_inline)) {
+    const unsigned base = lds0 + W_BASE + wstage * W_BYTES;
+#pragma unroll
+    for (int i = 0; i < W_INSTR; ++i)
+      if (i >= first && i < last)
+        copy16_to_lds(wbase, w_src[i] + static_cast<uint32_t>(kt0 + kt) * w_step, base + i * (NWAVES * 1024));
+  };
+
+  // 32-row blocks of this wavefront that hold rows of the group: the K loop is compiled for
+  // 0, MB/4, MB/2 and MB blocks and a wavefront runs the smallest that covers its own (every
+  // variant copies and synchronises alike).  The last row block of a group is mostly empty.
+  int live = (end - row0 - wm0 + 31) / 32;
+  live = live < 0 ? 0 : (live > MB ? MB : live);
+  live = __builtin_amdgcn_readfirstlane(live);
+
+  // a lane's fragment of a 32-row block for K half kh: 32 bytes = chunks 4 kh + 2 lhi, +1
+  auto read32 = [&](const char* tile, int row, int kh) __attribute__((always_inline)) -> i32x8 {
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(tile + kmajor_off(row, kh * 4 + lhi * 2));
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(tile + kmajor_off(row, kh * 4 + lhi * 2 + 1));
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  // unit u of a K step = K half (u >> 1), token-row half (u & 1)
+  auto read_unit_t = [&](int stage, int u, i32x8 (&tf)[HB], auto blocks) __attribute__((always_inline)) {
+    constexpr int LC = decltype(blocks)::value;
+    const char* at = smem + stage * A_BYTES;
+    const int kh = u >> 1, rh = u & 1;
+#pragma unroll
+    for (int mb = 0; mb < HB; ++mb)
+      if (rh * HB + mb < LC) tf[mb] = read32(at, wm0 + (rh * HB + mb) * 32 + l32, kh);
+  };
+  // column block `nb` of K half kh: block 0 before the unit of token-row half 0, block 1 at its
+  // start (a wavefront with at most HB live blocks has no other unit)
+  auto read_unit_w = [&](int wstage, int kh, int nb, i32x8 (&wf)[NB], auto blocks) __attribute__((always_inline)) {
+    constexpr int LC = decltype(blocks)::value;
+    if (LC == 0) return;
+    wf[nb] = read32(smem + W_BASE + wstage * W_BYTES, wn0 + nb * 32 + l32, kh);
+  };
+
+  f32x16 acc[MB][NB];
+  auto zero_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mb][nb][i] = 0.0f;
+  };
+  zero_acc();
+  auto multiply_unit = [&](int rh, i32x8 (&tf)[HB], i32x8 (&wf)[NB], auto blocks) __attribute__((always_inline)) {
+    constexpr int LC = decltype(blocks)::value;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+      for (int mb = 0; mb < HB; ++mb) {
+        if (rh == 0 && mb < LC)
+          acc[mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+              wf[nb], tf[mb], acc[mb][nb], 0 /* A: e4m3 */, 0 /* B: e4m3 */, 0, 127, 0, 127);
+        if (rh == 1 && HB + mb < LC)
+          acc[HB + mb][nb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
+              wf[nb], tf[mb], acc[HB + mb][nb], 0, 0, 0, 127, 0, 127);
+      }
+    }
+  };
+  // A unit reads 2 * (HB + 1) pieces of 16 bytes a lane for its HB * 2 MFMAs.  The empty asm
+  // statements tie the unit's accumulators to this point: an MFMA has no side effect, and the
+  // compiler otherwise sinks all sixteen of a K step below the (conditional) copy blocks, to
+  // the end of the step, with every fragment of the step live at once.
+  auto interleave_unit = [&](int rh, auto blocks) __attribute__((always_inline)) {
+    constexpr int LC = decltype(blocks)::value;
+#pragma unroll
+    for (int i = 0; i < HB * NB; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);  // two LDS reads
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int mb = 0; mb < HB; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        if (rh == 0 && mb < LC) asm volatile("" : "+v"(acc[mb][nb]));
+        if (rh == 1 && HB + mb < LC) asm volatile("" : "+v"(acc[HB + mb][nb]));
+      }
+  };
+
+  i32x8 tfA[HB], tfB[HB], wfP[NB], wfQ[NB];
+  // The accumulators of column tile `tile` leave through LDS regions that no copy in flight
+  // writes: wavefronts 0..3 through the token stage `a_free` (BM = 256; a spare region for
+  // BM = 128, whose token stages are too small), the others through the weight stage `w_free`.
+  constexpr int EPI_BYTES = epi_wave_bytes<NB, 32>();
+  constexpr int SPARE_BASE = W_BASE + 3 * W_BYTES;
+  const int row0_wg = row0, end_wg = end, lane_wg = lane;
+  auto store_acc = [&](int tile, int a_free, int w_free) __attribute__((always_inline)) {
+    const int64_t n0 = static_cast<int64_t>(nt0 + tile) * BN;
+    // (opaque copies: the rows are the same for every tile of the work item, and the compiler
+    // would otherwise keep the store's row addresses in registers across the K loop)
+    int row0 = row0_wg, end = end_wg, lane = lane_wg;
+    asm volatile("" : "+s"(row0), "+s"(end), "+v"(lane));
+    const int l32 = lane & 31, lhi = lane >> 5;
+    // dequantise: acc * a_scale[row] * w_scale[e, n], one run of four channel scales at a time
+    // (all eight float4 loads hoisted next to the 128 accumulators spilled 31-40 registers)
+    const float* wsc = fa.w_scale + static_cast<int64_t>(expert) * g.N;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int run = 0; run < 4; ++run) {
+        int64_t n = n0 + wn0 + nb * 32 + run * 8 + lhi * 4;
+        n = n + 3 < g.N ? n : g.N - 4;  // N is a multiple of 8; columns past N are not stored
+        const float4 ws = *reinterpret_cast<const float4*>(wsc + n);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          acc[mb][nb][run * 4 + 0] *= a_scale[mb] * ws.x;
+          acc[mb][nb][run * 4 + 1] *= a_scale[mb] * ws.y;
+          acc[mb][nb][run * 4 + 2] *= a_scale[mb] * ws.z;
+          acc[mb][nb][run * 4 + 3] *= a_scale[mb] * ws.w;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    if (lds_epilogue_ok<T>(g)) {
+      char* epi;
+      if (wave < NWAVES / 2)
+        epi = smem + (BM == 256 ? a_free * A_BYTES : SPARE_BASE) + wave * EPI_BYTES;
+      else
+        epi = smem + W_BASE + w_free * W_BYTES + (wave - NWAVES / 2) * EPI_BYTES;
+      store_tile_lds<T, ACT, MB, NB, 32>(g, acc, epi, row0, end, n0, wm0, wn0, lane);
+    } else {
+      store_tile<T, ACT, MB>(g, acc, row0, end, n0, wm0, wn0, l32, lhi);
+    }
+  };
+  auto main_loop = [&](auto blocks) __attribute__((always_inline)) {
+    const int S = ntiles * KT;   // K steps of this work item; step gs is step gs % KT of tile gs / KT
+    int kt_a = 0;                // copy cursors: K step (within its tile) to copy next
+    int kt_w = 0, tile_w = 0;
+    auto advance_a = [&]() __attribute__((always_inline)) { kt_a = kt_a + 1 == KT ? 0 : kt_a + 1; };
+    auto advance_w = [&]() __attribute__((always_inline)) {
+      if (++kt_w == KT) {
+        kt_w = 0;
+        if (++tile_w < ntiles) set_w_src(tile_w);
+      }
+    };
+    issue_token_copies(0, kt_a, 0, A_INSTR);
+    advance_a();
+    issue_weight_copies(0, kt_w, 0, W_INSTR);
+    advance_w();
+    if (S > 1) {
+      issue_weight_copies(1, kt_w, 0, W_INSTR);
+      advance_w();
+      wait_copies_keep_youngest_and_barrier<W_INSTR>();
+    } else {
+      wait_copies_and_barrier();
+    }
+    read_unit_t(0, 0, tfA, blocks);
+    read_unit_w(0, 0, 0, wfP, blocks);
+    int stage = 0, wcur = 0;  // token stage gs % 2, weight stage gs % 3
+    int kt = 0, tile = 0;
+    constexpr int AH = (A_INSTR + 1) / 2, WH = (W_INSTR + 1) / 2;
+    for (int gs = 0; gs < S; ++gs) {
+      const int wnext = wcur == 2 ? 0 : wcur + 1;
+      const int wahead = wnext == 2 ? 0 : wnext + 1;
+      const bool more = gs + 1 < S, ahead = gs + 2 < S;
+      const bool tile_ends = kt + 1 == KT;
+      if (more) issue_token_copies(stage ^ 1, kt_a, 0, AH);
+      __builtin_amdgcn_s_setprio(2);
+      __builtin_amdgcn_sched_barrier(0);
+      read_unit_w(wcur, 0, 1, wfP, blocks);
+      read_unit_t(stage, 1, tfB, blocks);
+      multiply_unit(0, tfA, wfP, blocks);
+      interleave_unit(0, blocks);
+      if (more) {
+        issue_token_copies(stage ^ 1, kt_a, AH, A_INSTR);
+        advance_a();
       }
       __builtin_amdgcn_sched_barrier(0);
+      read_unit_w(wcur, 1, 0, wfQ, blocks);
+      read_unit_t(stage, 2, tfA, blocks);
+      multiply_unit(1, tfB, wfP, blocks);
+      interleave_unit(1, blocks);
+      if (ahead) issue_weight_copies(wahead, kt_w, 0, WH);
+      __builtin_amdgcn_sched_barrier(0);
+      read_unit_w(wcur, 1, 1, wfQ, blocks);
+      read_unit_t(stage, 3, tfB, blocks);
+      multiply_unit(0, tfA, wfQ, blocks);
+      interleave_unit(0, blocks);
+      if (ahead) {
+        issue_weight_copies(wahead, kt_w, WH, W_INSTR);
+        advance_w();
+      }
+      __builtin_amdgcn_s_setprio(0);
+      if (more) {
+        // the token copies of step gs+1 and the weight copies of step gs+1 (issued a
+        // step earlier) must have landed; the weight copies of step gs+2 may still fly
+        if (ahead) wait_copies_keep_youngest_and_barrier<W_INSTR>();
+        else wait_copies_and_barrier();
+        // (the first fragments of a next tile are read after the store of this one:
+        // held across the store they would crowd the register file)
+        if (!tile_ends) {
+          read_unit_t(stage ^ 1, 0, tfA, blocks);
+          read_unit_w(wnext, 0, 0, wfP, blocks);
+        }
+      }
+      multiply_unit(1, tfB, wfQ, blocks);
+      interleave_unit(1, blocks);
+      if (tile_ends) {
+        // every wavefront is past the barrier above (or no later step exists and
+        // nothing is in flight): the stages of this step are free
+        if (!more) {
+          __syncthreads();
+          if (threadIdx.x == 0 && next.slot != nullptr) {
+            next.value = atomicAdd(next.slot, 1u);
+            next.drawn = true;
+          }
+        }
+        store_acc(tile, stage, wcur);
+        // (leaving here, instead of through the loop condition, tells the compiler that the
+        // accumulators are dead during the store: their registers are the store's to use)
+        if (!more) break;
+        {
+          __syncthreads();  // later steps copy into the stages just used for the store
+          zero_acc();
+          read_unit_t(stage ^ 1, 0, tfA, blocks);
+          read_unit_w(wnext, 0, 0, wfP, blocks);
+        }
+        kt = 0;
+        ++tile;
+      } else {
+        ++kt;
+      }
+      stage ^= 1;
+      wcur = wnext;
     }
+  };
+  if (live == 0) main_loop(std::integral_constant<int, 0>{});
+  else if (MB >= 4 && live <= MB / 4) main_loop(std::integral_constant<int, (MB >= 4 ? MB / 4 : MB / 2)>{});
+  else if (live <= MB / 2) main_loop(std::integral_constant<int, MB / 2>{});
+  else main_loop(std::integral_constant<int, MB>{});
+}
 
-  if (lds_epilogue_ok<T>(g)) {
+// One resident workgroup per compute unit draws work item ids from the tile queues of the
+// launch stream (gemm_mfma_dma.hip describes them: id 8j + q belongs to queue q, a workgroup
+// draws from the queue of its XCD first, word 8 counts the workgroups that are done and the
+// last one clears the set); without a queue set (a launch that is being captured) workgroup b
+// takes ids b, b + gridDim.x, ...
+struct Fp8KernelArgs {
+  Fp8Args fa;
+  Sched s;
+  unsigned* queue;
+};
+typedef __attribute__((address_space(4))) const Fp8KernelArgs* fp8_kernarg_ptr;
+
+template <typename T, int BM, int ACT>
+__global__ __launch_bounds__(kThreads) void m_grouped_fp8_kernel(Fp8KernelArgs ka) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  // (beside the tile descriptor that fp8_work_item keeps in the third weight stage)
+  int* const sh_next = reinterpret_cast<int*>(smem + 2 * (BM * 128) + 2 * (BN * 128)) + 8;
+  // hardware register XCC_ID: the XCD this workgroup runs on
+  const int home = __builtin_amdgcn_s_getreg((31 << 11) | 20) & (kNumXcd - 1);
+  int tried = 0;  // queues found empty so far, the home queue first
+  NextDraw next{nullptr, 0u, false};
+  int64_t static_id = blockIdx.x;
+  for (;;) {
+    // The arguments are read from the kernel argument segment again for every work item: held
+    // in scalar registers across them they crowd out what the K loop keeps there.
+    fp8_kernarg_ptr kp = (fp8_kernarg_ptr)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(kp));
+    const Fp8KernelArgs* const args = (const Fp8KernelArgs*)kp;
+    __syncthreads();  // every wavefront is done with the LDS of the work item before
+    if (threadIdx.x == 0 && args->queue == nullptr) {
+      *sh_next = static_id < args->s.wgs ? static_cast<int>(static_id) : -1;
+      static_id += gridDim.x;
+    } else if (threadIdx.x == 0) {
+      unsigned* const queue = args->queue;
+      const int total = static_cast<int>(args->s.wgs);
+      int id = -1;
+      while (tried < kNumXcd) {
+        const int q = (home + tried) & (kNumXcd - 1);
+        // (a draw made during the last store went to this same queue)
+        const unsigned got = next.drawn ? next.value : atomicAdd(&queue[q], 1u);
+        next.drawn = false;
+        const int64_t cand = static_cast<int64_t>(got) * kNumXcd + q;
+        if (cand < total) {
+          id = static_cast<int>(cand);
+          break;
+        }
+        ++tried;
+      }
+      *sh_next = id;
+      next.slot = tried < kNumXcd ? &queue[(home + tried) & (kNumXcd - 1)] : nullptr;
+    }
     __syncthreads();
-    store_tile_lds<T, ACT, MB, NB>(g, acc, smem + wave * epi_wave_bytes<NB>(), row0, end, n0, wm0,
-                                   wn0, lane);
-  } else {
-    store_tile<T, ACT, MB>(g, acc, row0, end, n0, wm0, wn0, l32, lhi);
+    const int id = __builtin_amdgcn_readfirstlane(*sh_next);
+    if (id < 0) break;
+    fp8_work_item<T, BM, ACT>(args->fa, args->s, id, next);
   }
+  // (every workgroup ends here: each queue runs dry after s.wgs / 8 draws)
+  if (threadIdx.x == 0 && ka.queue != nullptr) {
+    unsigned* const queue = ka.queue;
+    __threadfence();
+    if (atomicAdd(&queue[kNumXcd], 1u) == gridDim.x - 1) {
+      for (int q = 0; q <= kNumXcd; ++q) atomicExch(&queue[q], 0u);
+    }
+  }
+}
+
+template <auto Kernel>
+int launch_fp8_kernel(const Fp8Args& fa, const Sched& s, size_t lds, hipStream_t stream) {
+  static bool configured = false;
+  if (!configured) {
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         static_cast<int>(lds));
+    if (err != hipSuccess)
+      return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds, hipGetErrorString(err));
+    configured = true;
+  }
+  int cus = 0;
+  unsigned* queue = nullptr;
+  const int rc = tile_queue_set_of(stream, &queue, &cus);
+  if (rc != MOE_OK) return rc;
+  Fp8KernelArgs ka;
+  ka.fa = fa;
+  ka.s = s;
+  ka.queue = queue;
+  // (a multiple of the XCD count, so that ids taken in strides of the grid stay on their XCD)
+  unsigned wgs = static_cast<unsigned>(cus) / kNumXcd * kNumXcd;
+  if (wgs == 0) wgs = static_cast<unsigned>(cus);
+  if (s.wgs < wgs) wgs = static_cast<unsigned>(s.wgs);
+  Kernel<<<dim3(wgs), kThreads, lds, stream>>>(ka);
+  return MOE_OK;
 }
 
 template <typename T, int BM>
 int launch_fp8(const Fp8Args& fa, hipStream_t stream) {
   const MGemmArgs& g = fa.g;
-  Sched s = make_sched(g, BM);
+  // two column tiles a work item where that still leaves several rounds of work items
+  const int64_t tiles = ((g.P + BM - 1) / BM + g.E / 2) * ((g.N + BN - 1) / BN) * (g.ksplit < 1 ? 1 : g.ksplit);
+  Sched s = make_sched(g, BM, tiles >= 2048 ? 2 : 1);
   if (s.wgs > 0x7fffffff) return fail(MOE_ERR_UNSUPPORTED, "grid too large");
-  const size_t lds = 2 * (BM * 128) + 3 * (BN * 128);  // 2 token + 3 weight stages
-  const dim3 grid(static_cast<unsigned>(s.wgs));
+  // 2 token + 3 weight stages; BM = 128 adds room for the store staging of half the wavefronts
+  const size_t lds = 2 * (BM * 128) + 3 * (BN * 128) + (BM == 256 ? 0 : 4 * epi_wave_bytes<NB, 32>());
   MOE_DISPATCH_ACT(g.epilogue, ACT, {
-    auto kernel = m_grouped_fp8_kernel<T, BM, ACT>;
-    static bool configured = false;
-    if (!configured) {
-      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(lds));
-      if (err != hipSuccess)
-        return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds,
-                    hipGetErrorString(err));
-      configured = true;
-    }
-    kernel<<<grid, kThreads, lds, stream>>>(fa, s);
+    const int rc = launch_fp8_kernel<m_grouped_fp8_kernel<T, BM, ACT>>(fa, s, lds, stream);
+    if (rc != MOE_OK) return rc;
   });
   return check_launch("m_grouped_gemm_fp8");
 }
@@ -475,6 +724,17 @@ extern "C" int moe_m_grouped_gemm_fp8(const void* a, const float* a_scale, int64
                 "fp8 GEMM needs K %% 128 == 0, N %% 8 == 0, lda %% 16 == 0 and 16-byte aligned "
                 "operands (K=%lld N=%lld lda=%lld)",
                 (long long)K, (long long)N, (long long)lda);
+  // copy sources are a wave-uniform base and a 32-bit byte offset per lane: from the token matrix
+  // when its rows are gathered (from the first row of a block otherwise), from the weights of one
+  // expert (of one column tile when they are tile-major)
+  {
+    const int64_t limit = int64_t(1) << 32;
+    const int64_t a_span = (gather ? a_rows : 256) * lda + K;
+    const int64_t w_span = w_tiled ? (K / BKQ + 1) * (BN * BKQ) : N * K;
+    if (a_span >= limit || w_span >= limit)
+      return fail(MOE_ERR_UNSUPPORTED, "fp8 GEMM: a gathered token matrix and the weights of one expert "
+                  "must stay below 4 GiB (%lld and %lld bytes)", (long long)a_span, (long long)w_span);
+  }
   Fp8Args fa;
   fa.g = MGemmArgs{a,       a_rows, lda,     w,      N * K,         1,       K,         c,
                    c_rows,  ldc,    nullptr, 0,      group_indices, indices, idx_bytes, scales,

@@ -60,6 +60,10 @@ bool m_grouped_mfma_dma_supported(const MGemmArgs& g);  // K % 64 == 0, 16-byte 
 int launch_m_grouped_mfma_dma(const MGemmArgs& g, hipStream_t stream);
 bool k_grouped_mfma_supported(const KGemmArgs& g);
 int launch_k_grouped_mfma(const KGemmArgs& g, hipStream_t stream);
+// The tile-queue set of `stream` on the current device (16 words of a __device__ array that
+// the persistent GEMM kernels draw work item ids from; nullptr while the stream is being
+// captured: ids are then taken in strides of the grid) and the device's compute-unit count.
+int tile_queue_set_of(hipStream_t stream, unsigned** queue, int* cus);
 int launch_row_gather_kmajor(const void* src, int64_t src_rows, int64_t src_stride, const void* idx,
                              int idx_bytes, int idx_div, const int32_t* group_indices, int E,
                              int64_t P, void* dst, int64_t ld_dst, int64_t features, int dtype,

@@ -633,6 +633,10 @@ int launch_act(const MGemmArgs& g, hipStream_t stream) {
 
 }  // namespace
 
+int tile_queue_set_of(hipStream_t stream, unsigned** queue, int* cus) {
+  return queue_set_of(stream, queue, cus);
+}
+
 bool m_grouped_mfma_dma_supported(const MGemmArgs& g) {
   // stores through LDS only; copy sources are 32-bit byte offsets from the token matrix
   // and from the weight matrix of one expert
