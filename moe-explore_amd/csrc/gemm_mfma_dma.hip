@@ -502,6 +502,21 @@ __global__ __launch_bounds__(64 * WVM * WVN) void m_grouped_dma_kernel(DmaKernel
           break;
         }
         ++tried;
+        // A queue that has run dry stays dry for the rest of the launch: look at all the
+        // counters at once (one round trip) and pass over the dry ones, instead of finding
+        // each of them empty with an atomic of its own when the launch drains.
+        unsigned seen[kNumXcd];
+#pragma unroll
+        for (int i = 0; i < kNumXcd; ++i)
+          seen[i] = __hip_atomic_load(&queue[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        while (tried < kNumXcd) {
+          const int qq = (home + tried) & (kNumXcd - 1);
+          unsigned c = 0;
+#pragma unroll
+          for (int i = 0; i < kNumXcd; ++i) c = i == qq ? seen[i] : c;
+          if (static_cast<int64_t>(c) * kNumXcd + qq < total) break;
+          ++tried;
+        }
       }
       *sh_next = id;
       next.slot = tried < kNumXcd ? &queue[(home + tried) & (kNumXcd - 1)] : nullptr;
