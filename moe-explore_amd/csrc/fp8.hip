@@ -574,6 +574,19 @@ __global__ __launch_bounds__(kThreads) void m_grouped_fp8_kernel(Fp8KernelArgs k
           break;
         }
         ++tried;
+        // (a dry queue stays dry: one look at all counters passes over the other dry ones)
+        unsigned seen[kNumXcd];
+#pragma unroll
+        for (int i = 0; i < kNumXcd; ++i)
+          seen[i] = __hip_atomic_load(&queue[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        while (tried < kNumXcd) {
+          const int qq = (home + tried) & (kNumXcd - 1);
+          unsigned c = 0;
+#pragma unroll
+          for (int i = 0; i < kNumXcd; ++i) c = i == qq ? seen[i] : c;
+          if (static_cast<int64_t>(c) * kNumXcd + qq < total) break;
+          ++tried;
+        }
       }
       *sh_next = id;
       next.slot = tried < kNumXcd ? &queue[(home + tried) & (kNumXcd - 1)] : nullptr;
