@@ -278,6 +278,9 @@ MOE_API int moe_m_grouped_gemm_glu_bwd(const void* a, int64_t a_rows, int64_t ld
  * linear 32 KiB read and a column tile one sequential stream from HBM.
  * ksplit, c_split_stride: as for moe_m_grouped_gemm (K cut into parts that store to their
  * own copy of c; only without an activation, K % (128 * ksplit) == 0).
+ * MOE_ERR_UNSUPPORTED for K not a multiple of 128, N not a multiple of 8, rows that are not
+ * 16-byte aligned, and for a gathered token matrix (a_rows * lda bytes) or the weights of one
+ * expert (N * K bytes) of 4 GiB or more: the kernel addresses both with 32-bit offsets.
  */
 #define MOE_FP8_W_TILED 4
 MOE_API int moe_quantize_rows_fp8(const void* x, int64_t ldx, void* q, int64_t ldq, float* scale,

@@ -183,3 +183,62 @@ def test_fp8_gate_up_gemm_full_width_against_dequantised_oracle(config4_weights,
         wd = (codes.float() * q1.scale[e].unsqueeze(-1)).t().cpu()   # [K, N]
         ref = xd[ind[lo:hi] // k] @ wd
         assert_parity(h[lo:hi], ref, torch.bfloat16, f"fp8 gate/up GEMM, expert {e}", tol=1e-2)
+
+
+@pytest.mark.parametrize("tiled", [True, False])
+def test_fp8_many_tiles_odd_column_tile_count_one_k_step(tiled):
+    """More than 2048 tiles, so a work item takes two adjacent column tiles, with 65 column
+    tiles (the last work item of a row block has one) and K = 128 (one K step a tile: the
+    copies of a work item's second tile start before its first step is multiplied); through
+    the gather and the scatter."""
+    from moe_explore.expert_permute import get_token_indices
+    from moe_explore.fp8 import quantize_rows, quantize_expert_weights, m_grouped_gemm_fp8
+    g = seeded(65)
+    T, E, k, K, N = 4096, 8, 2, 128, 65 * 256
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    p = get_token_indices(idx.cuda(), k, E, zero_prefix=True)
+    x = randn((T, K), g, torch.bfloat16)
+    w = randn((E, K, N), g, torch.bfloat16, 0.05)
+    xq, xs = quantize_rows(x.cuda())
+    wq = quantize_expert_weights(w.cuda(), tiled=tiled)
+    xd = xq.cpu().float() * xs.cpu().unsqueeze(1)
+    wd = (wq.codes().cpu().float() * wq.scale.cpu().unsqueeze(-1)).transpose(1, 2)
+    perm, gi = p.indices.cpu(), p.group_indices.cpu()
+    out = m_grouped_gemm_fp8(xq, xs, wq, p.group_indices, p.indices, gather=True, num_tokens=T, topk=k)
+    ref = moe_ref.grouped_matmul_gather_scatter(xd, wd, gi, perm, gather=True, topk=k)
+    assert_parity(out, ref, torch.bfloat16, "fp8 gemm, gathered, 65 column tiles", tol=1e-2)
+    rows = out  # [T*k, N] in sorted order: feed them back through the scatter with a narrow weight
+    w2 = randn((E, N, 128), g, torch.bfloat16, 0.05)
+    aq, as_ = quantize_rows(rows)
+    w2q = quantize_expert_weights(w2.cuda(), tiled=tiled)
+    out2 = m_grouped_gemm_fp8(aq, as_, w2q, p.group_indices, p.indices, scatter=True, num_tokens=T, topk=k)
+    ad = aq.cpu().float() * as_.cpu().unsqueeze(1)
+    w2d = (w2q.codes().cpu().float() * w2q.scale.cpu().unsqueeze(-1)).transpose(1, 2)
+    ref2 = moe_ref.grouped_matmul_gather_scatter(ad, w2d, gi, perm, scatter=True, topk=k)
+    assert_parity(out2, ref2, torch.bfloat16, "fp8 gemm, scattered, K = 65 * 256", tol=1e-2)
+
+
+def test_fp8_operands_beyond_32_bit_offsets_are_refused():
+    """The copy sources are 32-bit offsets from the token matrix (when gathered) and from one
+    expert's weights: larger operands are refused before anything is launched (the sizes
+    below are only claimed, the buffers are small and never touched)."""
+    from moe_explore import _C
+    dev = "cuda"
+    buf = torch.zeros(4096, device=dev, dtype=torch.uint8)
+    scale = torch.ones(1024, device=dev, dtype=torch.float32)
+    gi = torch.zeros(3, device=dev, dtype=torch.int32)
+    idx = torch.zeros(16, device=dev, dtype=torch.int32)
+    lib = _C.load()
+
+    def call(a_rows, K, N, flags):
+        return lib.moe_m_grouped_gemm_fp8(
+            buf.data_ptr(), scale.data_ptr(), a_rows, K, buf.data_ptr(), scale.data_ptr(), buf.data_ptr(),
+            16, N, gi.data_ptr(), idx.data_ptr(), 4, 0, 2, K, N, 1, flags, 0, _C.dtype_code(torch.bfloat16),
+            1, 0, _C.stream_of(buf))
+    # gathered token matrix of 2^20 rows x 4096 bytes = 4 GiB
+    assert call(1 << 20, 4096, 256, _C.GEMM_GATHER_A) == -2  # MOE_ERR_UNSUPPORTED
+    # one expert's weights: 2^16 x 2^16 bytes
+    assert call(16, 1 << 16, 1 << 16, 0) == -2  # MOE_ERR_UNSUPPORTED
+    # within reach: group_indices are all zero, so nothing is computed
+    assert call(16, 128, 256, 0) == 0
+    torch.cuda.synchronize()
