@@ -307,7 +307,7 @@ MOE_API int moe_m_grouped_gemm_fp8(const void* a, const float* a_scale, int64_t 
  *   the order inside a token is unspecified there); logits_out [T, E] fp32 or NULL: the
  *   logits the scores were computed from, which moe_router_bwd takes.
  * x and w have the same 16-bit dtype (MFMA on 16-bit operands, fp32 accumulation), or w is
- * fp32 or both are (fp32 operands).  MOE_ERR_UNSUPPORTED for more than 256 experts,
+ * fp32 or both are (fp32 operands).  MOE_ERR_UNSUPPORTED for more than 512 experts,
  * top-k above 16, or x rows that cannot be read 16 bytes at a time.
  * Workspace: moe_router_workspace_bytes(d, E, x_dtype, w_dtype) bytes, 16-byte aligned (a
  * K-contiguous copy of w that the call writes first).

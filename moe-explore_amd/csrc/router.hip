@@ -30,7 +30,9 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 constexpr int kBlock = 32;    // tokens per MFMA row block; a workgroup owns MBW of them
 constexpr int kLpt = 8;       // lanes per token in the selection phase
 constexpr int kMaxTopk = 16;
-constexpr int kMaxExperts = 256;
+constexpr int kChunk = 256;       // experts a wavefront accumulates (8 blocks of 32)
+constexpr int kMaxExperts = 512;   // two chunks, handled by different wavefronts (with four the
+                                   // selection phase, 8 lanes a token, takes longer than ATen's kernels)
 
 struct RouterArgs {
   const void* x;
@@ -93,21 +95,27 @@ __device__ __forceinline__ float4 load4_as_f32(const TX* p) {
 }
 
 // F32: operands and MFMA in fp32 (wt is float); otherwise wt has the type of x.
-// NB: 32-expert blocks.  MBW: 32-token blocks of a workgroup (every weight fragment is
-// used MBW times; only 1 is instantiated).  U: K steps whose loads are issued together.
-template <typename TX, bool F32, int NB, int MBW, int U>
+// NB: 32-expert blocks a wavefront accumulates.  EC: chunks of NB * 32 experts; with more
+// than one, wavefront w works on chunk w % EC and the wavefronts of a chunk split K (more
+// than 256 experts: NB = 8, EC = 2).  MBW: 32-token blocks of a workgroup (every weight
+// fragment is used MBW times; only 1 is instantiated).  U: K steps whose loads are issued
+// together.  Dynamic LDS: the logits of the workgroup's tokens, kBlock * MBW * (EC * NB * 32 + 1)
+// floats.
+template <typename TX, bool F32, int NB, int MBW, int U, int EC = 1>
 __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
   constexpr int KSTEP = F32 ? 8 : 16;  // K consumed per step: a 16-byte load per lane and operand
-  constexpr int EP = NB * 32;
+  constexpr int EP = EC * NB * 32;
   constexpr int PITCH = EP + 1;
   constexpr int kTokens = kBlock * MBW;
-  __shared__ float logits[kTokens * PITCH];
+  extern __shared__ float logits[];
   __shared__ int sel_s[kBlock][kMaxTopk];  // per token of the block being selected
   __shared__ float val_s[kBlock][kMaxTopk];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int nwaves = blockDim.x >> 6;
+  const int nwaves = (blockDim.x >> 6) / EC;  // wavefronts that split K for one chunk of experts
+  const int chunk = EC == 1 ? 0 : wave % EC;
+  const int kwave = EC == 1 ? wave : wave / EC;
   const int l32 = lane & 31, lhi = lane >> 5;
   const int64_t t0 = static_cast<int64_t>(blockIdx.x) * kTokens;
 
@@ -122,7 +130,7 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
   // K steps [s_begin, s_end) of this wavefront
   const int steps = static_cast<int>(g.dpad / KSTEP);
   const int per_wave = (steps + nwaves - 1) / nwaves;
-  const int s_begin = wave * per_wave;
+  const int s_begin = kwave * per_wave;
   const int s_end = s_begin + per_wave < steps ? s_begin + per_wave : steps;
 
   const TX* xrow[MBW];
@@ -136,7 +144,7 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
   const CT* wrow[NB];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb) {
-    int e = nb * 32 + l32;
+    int e = chunk * (NB * 32) + nb * 32 + l32;
     e = e < g.E ? e : g.E - 1;
     wrow[nb] = static_cast<const CT*>(g.wt) + static_cast<int64_t>(e) * g.dpad;
   }
@@ -193,8 +201,9 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
 
   // ---- add the partial logits of the wavefronts, in wavefront order -----------------
   // accumulator element run*4 + j of block nb: token l32, expert nb*32 + run*8 + lhi*4 + j
+  // (the wavefronts of different chunks write different columns)
   for (int w = 0; w < nwaves; ++w) {
-    if (wave == w) {
+    if (kwave == w) {
 #pragma unroll
       for (int mb = 0; mb < MBW; ++mb)
 #pragma unroll
@@ -203,7 +212,7 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
           for (int r = 0; r < 4; ++r)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              float* p = &logits[(mb * kBlock + l32) * PITCH + nb * 32 + r * 8 + lhi * 4 + j];
+              float* p = &logits[(mb * kBlock + l32) * PITCH + chunk * (NB * 32) + nb * 32 + r * 8 + lhi * 4 + j];
               *p = (w == 0 ? 0.0f : *p) + acc[mb][nb][r * 4 + j];
             }
     }
@@ -257,20 +266,26 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
   }
 
   // top-k: each round, every lane offers its best remaining expert (ties: lowest id)
-  uint32_t taken = 0;  // bit i: expert q + kLpt*i
+  uint32_t taken[EC];  // word c, bit b: expert q + kLpt * (32 c + b)
+#pragma unroll
+  for (int c = 0; c < EC; ++c) taken[c] = 0;
   int* sel = sel_s[tid / kLpt];
   float* val = val_s[tid / kLpt];
 #pragma unroll 1
   for (int j = 0; j < topk; ++j) {
     float best = 0.0f;
     int best_e = -1;
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+      const uint32_t tk = taken[c];
 #pragma unroll 1
-    for (int i = 0, e = q; e < E; ++i, e += kLpt) {
-      if (taken & (1u << i)) continue;
-      const float key = ernie ? row[e] + g.bias[e] : row[e];
-      if (best_e < 0 || key > best) {
-        best = key;
-        best_e = e;
+      for (int b = 0, e = q + kLpt * 32 * c; b < 32 && e < E; ++b, e += kLpt) {
+        if (tk & (1u << b)) continue;
+        const float key = ernie ? row[e] + g.bias[e] : row[e];
+        if (best_e < 0 || key > best) {
+          best = key;
+          best_e = e;
+        }
       }
     }
 #pragma unroll
@@ -282,7 +297,12 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
       best_e = take ? oe : best_e;
     }
     best_e = best_e < 0 ? 0 : best_e;  // only if topk > E, which the entry point rejects
-    if (best_e % kLpt == q) taken |= 1u << (best_e / kLpt);
+    if (best_e % kLpt == q) {
+      const int i = best_e / kLpt;
+#pragma unroll
+      for (int c = 0; c < EC; ++c)
+        if ((i >> 5) == c) taken[c] |= 1u << (i & 31);
+    }
     if (q == 0) {
       sel[j] = best_e;
       val[j] = row[best_e];
@@ -438,11 +458,28 @@ int launch_fwd(const RouterArgs& g, hipStream_t stream) {
   const int nb = (g.E + 31) / 32;
   const int64_t wgs = (g.T + kBlock - 1) / kBlock;
   const dim3 grid(static_cast<unsigned>(wgs));
-  const dim3 block(64 * (wgs >= 2048 ? 4 : 8));
-  if (nb <= 1) router_fwd_kernel<TX, F32, 1, 1, 16><<<grid, block, 0, stream>>>(g);
-  else if (nb <= 2) router_fwd_kernel<TX, F32, 2, 1, 8><<<grid, block, 0, stream>>>(g);
-  else if (nb <= 4) router_fwd_kernel<TX, F32, 4, 1, 4><<<grid, block, 0, stream>>>(g);
-  else router_fwd_kernel<TX, F32, 8, 1, 2><<<grid, block, 0, stream>>>(g);
+  const dim3 block(64 * (wgs >= 2048 && g.E <= kChunk ? 4 : 8));
+  auto lds_bytes = [](int experts) { return static_cast<size_t>(kBlock) * (experts + 1) * sizeof(float); };
+  if (nb <= 1) router_fwd_kernel<TX, F32, 1, 1, 16><<<grid, block, lds_bytes(32), stream>>>(g);
+  else if (nb <= 2) router_fwd_kernel<TX, F32, 2, 1, 8><<<grid, block, lds_bytes(64), stream>>>(g);
+  else if (nb <= 4) router_fwd_kernel<TX, F32, 4, 1, 4><<<grid, block, lds_bytes(128), stream>>>(g);
+  else if (nb <= 8) router_fwd_kernel<TX, F32, 8, 1, 2><<<grid, block, lds_bytes(256), stream>>>(g);
+  else {
+    // more than 256 experts: two chunks of 256, eight wavefronts; the logits of the 32
+    // tokens need more than the 64 KiB of LDS a kernel gets without asking
+    auto launch = [&](auto kernel, int experts) -> int {
+      const size_t lds = lds_bytes(experts);
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 static_cast<int>(lds));
+      if (err != hipSuccess)
+        return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds, hipGetErrorString(err));
+      kernel<<<grid, block, lds, stream>>>(g);
+      return MOE_OK;
+    };
+    const int rc = launch(router_fwd_kernel<TX, F32, 8, 1, 2, 2>, 512);
+    if (rc != MOE_OK) return rc;
+  }
   return check_launch("router (fused logits, softmax, top-k)");
 }
 

@@ -3,7 +3,7 @@
 On the GPU ``topk_router`` and ``ernie_router`` run as one fused HIP kernel (logits,
 fp32 softmax, top-k, renormalisation, cast) with a second small kernel for the gradient
 of the scores with respect to the logits; the two skinny matmuls of the backward pass
-stay on ATen.  Shapes outside the kernel's reach (more than 256 experts, top-k above 16,
+stay on ATen.  Shapes outside the kernel's reach (more than 512 experts, top-k above 16,
 rows that cannot be read 16 bytes at a time) and CPU tensors take the ATen formulation
 below, which is the reference's own.
 """
@@ -44,7 +44,7 @@ def _fused_supported(x, weight, topk, ernie):
     d, E = weight.shape
     f32 = torch.float32 in (x.dtype, weight.dtype)
     vec = 4 if f32 else 8
-    return (x.size(1) == d and 0 < E <= 256 and 1 <= topk <= min(E, 16) and d % vec == 0
+    return (x.size(1) == d and 0 < E <= 512 and 1 <= topk <= min(E, 16) and d % vec == 0
             and x.stride(1) == 1 and x.stride(0) % vec == 0
             and x.data_ptr() % (vec * x.element_size()) == 0)
 

@@ -17,6 +17,8 @@ pytestmark = pytest.mark.gpu
 # (T, d, E, topk)
 SHAPES = [(512, 256, 8, 2), (1000, 512, 64, 8), (96, 1024, 128, 8), (70, 264, 256, 16),
           (33, 72, 5, 3), (2048, 2048, 64, 6), (64, 128, 4, 4), (1, 64, 8, 2)]
+# more than 256 experts: two chunks of 256 handled by different wavefronts
+MANY_EXPERTS = [(200, 512, 384, 8), (100, 1024, 512, 16), (77, 256, 500, 6), (130, 2048, 320, 8), (40, 512, 257, 4)]
 
 
 def _inputs(T, d, E, dtype, seed, w_dtype=None):
@@ -89,6 +91,43 @@ def test_topk_router_matches_oracle(shape, dtype, softmax_first, normalize):
     # the oracle's own entry point agrees with the reading of it above
     so, io = moe_ref.topk_router(x.float(), w.float(), topk, softmax_first, normalize)
     assert so.shape == s.shape and io.shape == i.shape
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", MANY_EXPERTS)
+@pytest.mark.parametrize("softmax_first,normalize", [(True, True), (False, False)])
+def test_topk_router_more_than_256_experts(shape, dtype, softmax_first, normalize):
+    from moe_explore.params import TopkRouterParams
+    from moe_explore.router import topk_router, _fused_supported
+    T, d, E, topk = shape
+    x, w = _inputs(T, d, E, dtype, seed=T + E)
+    assert _fused_supported(x.cuda(), w.cuda(), topk, False)
+    s, i = topk_router(x.cuda(), TopkRouterParams(w.cuda(), topk, softmax_first, normalize))
+    _check(s.cpu(), i.cpu(), x, w, topk, softmax_first, normalize)
+
+
+def test_ernie_router_and_backward_with_384_experts():
+    """The bias path, the saved logits and the gradient of the scores with 384 experts."""
+    from moe_explore.params import ErnieRouterParams, TopkRouterParams
+    from moe_explore.router import ernie_router, topk_router
+    T, d, E, topk = 150, 512, 384, 8
+    x, w = _inputs(T, d, E, torch.bfloat16, seed=384, w_dtype=torch.float32)
+    bias = torch.randn(E, generator=seeded(5)) * 0.01
+    s, i = ernie_router(x.cuda(), ErnieRouterParams(w.cuda(), bias.cuda(), topk))
+    _check(s.cpu(), i.cpu(), x, w, topk, True, True, bias=bias)
+    xg = x.float().clone().cuda().requires_grad_(True)
+    wg = w.clone().cuda().requires_grad_(True)
+    sg, ig = topk_router(xg, TopkRouterParams(wg, topk, True, True))
+    g = torch.randn(sg.shape, generator=seeded(6))
+    sg.backward(g.cuda())
+    xr = x.float().clone().requires_grad_(True)
+    wr = w.clone().requires_grad_(True)
+    pr = torch.softmax(xr @ wr, -1)
+    sr = torch.gather(pr, 1, ig.cpu())
+    sr = sr / sr.sum(-1, keepdim=True)
+    sr.backward(g)
+    assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 1e-4
+    assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= 1e-4
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
