@@ -165,10 +165,17 @@ def main():
     if args.only == "copy":
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
+        dst.copy_(src)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
         for _ in range(args.steps):
             dst.copy_(src)
+        end.record()
         torch.cuda.synchronize()
-        print("copied 1 GiB x %d" % args.steps)
+        ms = start.elapsed_time(end) / args.steps
+        # (what a plain device copy reaches is the practical roof of the HBM-bound passes)
+        print("copied 1 GiB x %d: %.3f ms a copy = %.0f GB/s read + written (%.2f of 8 TB/s)"
+              % (args.steps, ms, 2 * (1 << 30) / ms / 1e6, 2 * (1 << 30) / ms / 1e6 / 8000))
         return
     if args.only == "ablation":
         from moe_explore.hip_kernels.row_gather_scatter import row_gather_kmajor
