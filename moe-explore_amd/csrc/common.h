@@ -25,6 +25,10 @@ void clear_error();
 // compute units of the current device (cached); -1 with the error set on failure
 int num_cus();
 
+// Lets `kernel` be launched with `bytes` of dynamic LDS (more than the 64 KiB a kernel gets
+// without asking); set once per kernel and device.  Always called with the same size for a kernel.
+int allow_dynamic_lds(const void* kernel, size_t bytes);
+
 inline int check_launch(const char* what) {
   hipError_t err = hipGetLastError();
   if (err != hipSuccess) return fail(MOE_ERR_HIP, "%s: %s", what, hipGetErrorString(err));

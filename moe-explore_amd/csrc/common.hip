@@ -4,6 +4,10 @@
 #include <stdarg.h>
 #include <stdio.h>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 namespace moe {
 namespace {
 thread_local char g_error[512] = "";
@@ -32,6 +36,21 @@ int num_cus() {
     return fail(MOE_ERR_HIP, "hipDeviceGetAttribute(multiprocessor count): %s", hipGetErrorString(err)), -1;
   if (dev >= 0 && dev < kMaxDevices) cached[dev] = n;
   return n;
+}
+
+int allow_dynamic_lds(const void* kernel, size_t bytes) {
+  static std::mutex lock;
+  static std::set<std::pair<const void*, int>> done;
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return fail(MOE_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(err));
+  std::lock_guard<std::mutex> hold(lock);
+  if (done.find({kernel, dev}) != done.end()) return MOE_OK;
+  err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes));
+  if (err != hipSuccess)
+    return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", bytes, hipGetErrorString(err));
+  done.insert({kernel, dev});
+  return MOE_OK;
 }
 
 }  // namespace moe

@@ -608,18 +608,11 @@ __global__ __launch_bounds__(kThreads) void m_grouped_fp8_kernel(Fp8KernelArgs k
 
 template <auto Kernel>
 int launch_fp8_kernel(const Fp8Args& fa, const Sched& s, size_t lds, hipStream_t stream) {
-  static bool configured = false;
-  if (!configured) {
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(lds));
-    if (err != hipSuccess)
-      return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds, hipGetErrorString(err));
-    configured = true;
-  }
+  int rc = allow_dynamic_lds(reinterpret_cast<const void*>(Kernel), lds);
+  if (rc != MOE_OK) return rc;
   int cus = 0;
   unsigned* queue = nullptr;
-  const int rc = tile_queue_set_of(stream, &queue, &cus);
+  rc = tile_queue_set_of(stream, &queue, &cus);
   if (rc != MOE_OK) return rc;
   Fp8KernelArgs ka;
   ka.fa = fa;

@@ -673,25 +673,9 @@ int launch_k_grouped_mfma(const KGemmArgs& g, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>(wanted < cus ? wanted : cus));
   const int total = static_cast<int>(ntiles);
   constexpr size_t lds = KLDS_BYTES;
-  // (the six instantiations share one function-pointer type, so a flag inside a generic lambda
-  // would be shared as well: the attribute is set per kernel and per device, once)
   auto launch = [&](auto kernel) -> int {
-    static std::mutex lock;
-    static std::set<std::pair<const void*, int>> configured;
-    int dev = 0;
-    hipError_t err = hipGetDevice(&dev);
-    if (err != hipSuccess) return fail(MOE_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(err));
-    const void* fn = reinterpret_cast<const void*>(kernel);
-    {
-      std::lock_guard<std::mutex> hold(lock);
-      if (configured.find({fn, dev}) == configured.end()) {
-        err = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
-        if (err != hipSuccess)
-          return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds,
-                      hipGetErrorString(err));
-        configured.insert({fn, dev});
-      }
-    }
+    const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lds);
+    if (rc != MOE_OK) return rc;
     kernel<<<grid, kThreads, lds, stream>>>(g, s, total);
     return MOE_OK;
   };

@@ -244,16 +244,8 @@ int launch_act(const MGemmArgs& g, hipStream_t stream) {
   const dim3 grid(static_cast<unsigned>(s.wgs));
   MOE_DISPATCH_ACT(g.epilogue, ACT, {
     auto kernel = m_grouped_mfma_kernel<T, BM, WL, ACT>;
-    static bool configured = false;
-    if (!configured) {
-      hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           static_cast<int>(lds));
-      if (err != hipSuccess)
-        return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds,
-                    hipGetErrorString(err));
-      configured = true;
-    }
+    const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lds);
+    if (rc != MOE_OK) return rc;
     kernel<<<grid, kThreads, lds, stream>>>(g, s);
   });
   return check_launch("m_grouped_gemm (MFMA kernel)");

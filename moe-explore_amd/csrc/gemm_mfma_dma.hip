@@ -582,24 +582,16 @@ int queue_set_of(hipStream_t stream, unsigned** queue, int* cus) {
   return MOE_OK;
 }
 
-// Sets the kernel's dynamic LDS limit on first use and launches it with one workgroup per
+// Sets the kernel's dynamic LDS limit on first use (per device) and launches it with one workgroup per
 // compute unit (fewer if there are fewer work items).
 template <auto Kernel>
 int launch_kernel(const MGemmArgs& g, const Sched& s, dim3 grid, int threads, size_t lds,
                   hipStream_t stream) {
-  static bool configured = false;
-  if (!configured) {
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         static_cast<int>(lds));
-    if (err != hipSuccess)
-      return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds,
-                  hipGetErrorString(err));
-    configured = true;
-  }
+  int rc = allow_dynamic_lds(reinterpret_cast<const void*>(Kernel), lds);
+  if (rc != MOE_OK) return rc;
   int cus = 0;
   unsigned* queue = nullptr;
-  const int rc = queue_set_of(stream, &queue, &cus);
+  rc = queue_set_of(stream, &queue, &cus);
   if (rc != MOE_OK) return rc;
   DmaKernelArgs ka;
   ka.g = g;

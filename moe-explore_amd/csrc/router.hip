@@ -469,11 +469,8 @@ int launch_fwd(const RouterArgs& g, hipStream_t stream) {
     // tokens need more than the 64 KiB of LDS a kernel gets without asking
     auto launch = [&](auto kernel, int experts) -> int {
       const size_t lds = lds_bytes(experts);
-      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 static_cast<int>(lds));
-      if (err != hipSuccess)
-        return fail(MOE_ERR_HIP, "hipFuncSetAttribute(%zu bytes of LDS): %s", lds, hipGetErrorString(err));
+      const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lds);
+      if (rc != MOE_OK) return rc;
       kernel<<<grid, block, lds, stream>>>(g);
       return MOE_OK;
     };
