@@ -99,9 +99,10 @@ __device__ __forceinline__ float4 load4_as_f32(const TX* p) {
 // than one, wavefront w works on chunk w % EC and the wavefronts of a chunk split K (more
 // than 256 experts: NB = 8, EC = 2).  MBW: 32-token blocks of a workgroup (every weight
 // fragment is used MBW times; only 1 is instantiated).  U: K steps whose loads are issued
-// together.  Dynamic LDS: the logits of the workgroup's tokens, kBlock * MBW * (EC * NB * 32 + 1)
+// together.  LPT: lanes that share a token in the selection phase (8, or 16 with eight
+// wavefronts and more than 64 experts, where the selection is most of the kernel).  Dynamic LDS: the logits of the workgroup's tokens, kBlock * MBW * (EC * NB * 32 + 1)
 // floats.
-template <typename TX, bool F32, int NB, int MBW, int U, int EC = 1>
+template <typename TX, bool F32, int NB, int MBW, int U, int EC = 1, int LPT = kLpt>
 __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
   constexpr int KSTEP = F32 ? 8 : 16;  // K consumed per step: a 16-byte load per lane and operand
   constexpr int EP = EC * NB * 32;
@@ -219,12 +220,12 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
     __syncthreads();
   }
 
-  // ---- softmax, top-k, renormalisation: kLpt lanes per token ---------------------------
-  if (tid >= kBlock * kLpt) return;
-  const int q = tid % kLpt;
+  // ---- softmax, top-k, renormalisation: LPT lanes per token ---------------------------
+  if (tid >= kBlock * LPT) return;
+  const int q = tid % LPT;
 #pragma unroll 1
   for (int mb = 0; mb < MBW; ++mb) {
-  const int tt = mb * kBlock + tid / kLpt;
+  const int tt = mb * kBlock + tid / LPT;
   const int64_t t = t0 + tt;
   float* row = &logits[tt * PITCH];
   const int E = g.E, topk = g.topk;
@@ -234,19 +235,19 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
 
   auto group_max = [&](float v) __attribute__((always_inline)) {
 #pragma unroll
-    for (int o = 1; o < kLpt; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    for (int o = 1; o < LPT; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
     return v;
   };
   auto group_sum = [&](float v) __attribute__((always_inline)) {
 #pragma unroll
-    for (int o = 1; o < kLpt; o <<= 1) v += __shfl_xor(v, o, 64);
+    for (int o = 1; o < LPT; o <<= 1) v += __shfl_xor(v, o, 64);
     return v;
   };
 
   // the reference's logits are a matmul result in the dtype of x (router.py:22); the
   // Ernie router keeps them in fp32 (:44)
   float mx = -INFINITY;
-  for (int e = q; e < E; e += kLpt) {
+  for (int e = q; e < E; e += LPT) {
     float v = row[e];
     if (!ernie && sizeof(TX) == 2) v = to_f32(from_f32<TX>(v));
     row[e] = v;
@@ -256,30 +257,31 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
   mx = group_max(mx);
   if (softmax_first) {
     float z = 0.0f;
-    for (int e = q; e < E; e += kLpt) {
+    for (int e = q; e < E; e += LPT) {
       const float p = expf(row[e] - mx);
       row[e] = p;
       z += p;
     }
     z = group_sum(z);
-    for (int e = q; e < E; e += kLpt) row[e] = row[e] / z;
+    for (int e = q; e < E; e += LPT) row[e] = row[e] / z;
   }
 
   // top-k: each round, every lane offers its best remaining expert (ties: lowest id)
-  uint32_t taken[EC];  // word c, bit b: expert q + kLpt * (32 c + b)
+  constexpr int TW = (EP + 32 * LPT - 1) / (32 * LPT);
+  uint32_t taken[TW];  // word c, bit b: expert q + LPT * (32 c + b)
 #pragma unroll
-  for (int c = 0; c < EC; ++c) taken[c] = 0;
-  int* sel = sel_s[tid / kLpt];
-  float* val = val_s[tid / kLpt];
+  for (int c = 0; c < TW; ++c) taken[c] = 0;
+  int* sel = sel_s[tid / LPT];
+  float* val = val_s[tid / LPT];
 #pragma unroll 1
   for (int j = 0; j < topk; ++j) {
     float best = 0.0f;
     int best_e = -1;
 #pragma unroll
-    for (int c = 0; c < EC; ++c) {
+    for (int c = 0; c < TW; ++c) {
       const uint32_t tk = taken[c];
 #pragma unroll 1
-      for (int b = 0, e = q + kLpt * 32 * c; b < 32 && e < E; ++b, e += kLpt) {
+      for (int b = 0, e = q + LPT * 32 * c; b < 32 && e < E; ++b, e += LPT) {
         if (tk & (1u << b)) continue;
         const float key = ernie ? row[e] + g.bias[e] : row[e];
         if (best_e < 0 || key > best) {
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
       }
     }
 #pragma unroll
-    for (int o = 1; o < kLpt; o <<= 1) {
+    for (int o = 1; o < LPT; o <<= 1) {
       const float ob = __shfl_xor(best, o, 64);
       const int oe = __shfl_xor(best_e, o, 64);
       const bool take = oe >= 0 && (best_e < 0 || ob > best || (ob == best && oe < best_e));
@@ -297,10 +299,10 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
       best_e = take ? oe : best_e;
     }
     best_e = best_e < 0 ? 0 : best_e;  // only if topk > E, which the entry point rejects
-    if (best_e % kLpt == q) {
-      const int i = best_e / kLpt;
+    if (best_e % LPT == q) {
+      const int i = best_e / LPT;
 #pragma unroll
-      for (int c = 0; c < EC; ++c)
+      for (int c = 0; c < TW; ++c)
         if ((i >> 5) == c) taken[c] |= 1u << (i & 31);
     }
     if (q == 0) {
@@ -333,7 +335,7 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
     TX* so = static_cast<TX*>(g.scores) + t * topk;
     int64_t* io = g.idx + t * topk;
 #pragma unroll 1
-    for (int j = q; j < topk; j += kLpt) {
+    for (int j = q; j < topk; j += LPT) {
       const float v = normalize ? score(j) / sum : score(j);
       so[j] = from_f32<TX>(v);
       io[j] = sel[j];
@@ -462,7 +464,9 @@ int launch_fwd(const RouterArgs& g, hipStream_t stream) {
   auto lds_bytes = [](int experts) { return static_cast<size_t>(kBlock) * (experts + 1) * sizeof(float); };
   if (nb <= 1) router_fwd_kernel<TX, F32, 1, 1, 16><<<grid, block, lds_bytes(32), stream>>>(g);
   else if (nb <= 2) router_fwd_kernel<TX, F32, 2, 1, 8><<<grid, block, lds_bytes(64), stream>>>(g);
+  else if (nb <= 4 && block.x == 512) router_fwd_kernel<TX, F32, 4, 1, 4, 1, 16><<<grid, block, lds_bytes(128), stream>>>(g);
   else if (nb <= 4) router_fwd_kernel<TX, F32, 4, 1, 4><<<grid, block, lds_bytes(128), stream>>>(g);
+  else if (nb <= 8 && block.x == 512) router_fwd_kernel<TX, F32, 8, 1, 2, 1, 16><<<grid, block, lds_bytes(256), stream>>>(g);
   else if (nb <= 8) router_fwd_kernel<TX, F32, 8, 1, 2><<<grid, block, lds_bytes(256), stream>>>(g);
   else {
     // more than 256 experts: two chunks of 256, eight wavefronts; the logits of the 32
@@ -474,7 +478,7 @@ int launch_fwd(const RouterArgs& g, hipStream_t stream) {
       kernel<<<grid, block, lds, stream>>>(g);
       return MOE_OK;
     };
-    const int rc = launch(router_fwd_kernel<TX, F32, 8, 1, 2, 2>, 512);
+    const int rc = launch(router_fwd_kernel<TX, F32, 8, 1, 2, 2, 16>, 512);
     if (rc != MOE_OK) return rc;
   }
   return check_launch("router (fused logits, softmax, top-k)");
