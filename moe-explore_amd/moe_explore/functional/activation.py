@@ -36,6 +36,16 @@ def is_glu(act):
     return name is not None and "glu" in name
 
 
+def glu_form(act):
+    """Activation of a gated record (``GLUParams`` / ``GLUInterleavedParams``, ``params.py:16-27``)
+    given as the model's ``hidden_act``: "silu" means SwiGLU and "gelu" GeGLU, the rule of the
+    reference's ``tests/test_hf.py:61-64``; GLU names pass through."""
+    name = activation_name(act)
+    if name is None or is_glu(name):
+        return act
+    return "geglu" if name == "gelu" else "swiglu"
+
+
 def activation(x: torch.Tensor, activation: "Activation | str"):
     name = activation_name(activation)
     assert name in _NAMES, f"Invalid activation: {activation}"

@@ -16,7 +16,7 @@ import torch
 
 from moe_explore.params import MOEParams, MLPParams, GLUParams, GLUInterleavedParams
 from moe_explore.tracing import scope
-from moe_explore.functional.activation import activation, activation_name, is_glu
+from moe_explore.functional.activation import activation, activation_name, glu_form, is_glu
 from moe_explore.functional.scale_and_reduce import scale_and_reduce
 from moe_explore.router import router
 from moe_explore.expert_permute import get_token_indices
@@ -47,7 +47,7 @@ def to_interleaved(ep):
     comes back in the same interleaved layout and nothing is copied per step."""
     if isinstance(ep, GLUParams):
         return GLUInterleavedParams(interleave_glu_weights(ep.gate_weight, ep.up_weight),
-                                    ep.down_weight, ep.activation)
+                                    ep.down_weight, glu_form(ep.activation))
     return ep
 
 
@@ -94,14 +94,14 @@ def expert_weights(ep):
     if isinstance(ep, MLPParams):
         return ep.weight1, ep.weight2, ep.activation
     if isinstance(ep, GLUInterleavedParams):
-        return ep.interleaved_weight, ep.down_weight, ep.activation
+        return ep.interleaved_weight, ep.down_weight, glu_form(ep.activation)
     if isinstance(ep, GLUParams):
         gate, up = ep.gate_weight, ep.up_weight
         if torch.is_grad_enabled() and (gate.requires_grad or up.requires_grad):
             w1 = _InterleaveFunction.apply(gate, up)
         else:
             w1 = _cached_interleave(gate, up)
-        return w1, ep.down_weight, ep.activation
+        return w1, ep.down_weight, glu_form(ep.activation)
     raise ValueError(f"Unsupported expert parameter type: {type(ep)}")
 
 

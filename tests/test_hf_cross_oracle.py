@@ -187,3 +187,66 @@ def test_experts_match_transformers_experts_bf16(kind):
     with torch.no_grad():
         ref = blk.experts(x.float(), idx.cpu(), scores.float().cpu())
     assert_parity(out, ref, torch.bfloat16, f"{kind} experts, bf16", tol=2e-2)
+
+
+def _hf_case(model, hidden, inter, E, k, dev, dtype):
+    """(config, MOEParams, forward function of moe_explore.hf_moe_reference) of one model family;
+    the expert record carries the model's hidden_act ("silu"), as the reference's test builds it."""
+    from moe_explore import hf_moe_reference as hf
+    from moe_explore.params import MOEParams
+    from moe_explore.testing import random_ernie_router, random_glu, random_topk_router
+    experts = random_glu(E, hidden, inter, "silu", dev, dtype)
+    if model == "olmoe":
+        from transformers.models.olmoe.configuration_olmoe import OlmoeConfig
+        cfg = OlmoeConfig(hidden_size=hidden, intermediate_size=inter, num_experts=E,
+                          num_experts_per_tok=k, norm_topk_prob=False, hidden_act="silu")
+        router, forward = random_topk_router(E, hidden, k, True, False, dev, dtype), hf.olmoe_forward
+    elif model == "qwen3":
+        from transformers.models.qwen3_moe.configuration_qwen3_moe import Qwen3MoeConfig
+        cfg = Qwen3MoeConfig(hidden_size=hidden, moe_intermediate_size=inter, intermediate_size=inter,
+                             num_experts=E, num_experts_per_tok=k, norm_topk_prob=True, hidden_act="silu")
+        router, forward = random_topk_router(E, hidden, k, True, True, dev, dtype), hf.qwen3_moe_forward
+    else:
+        from transformers.models.ernie4_5_moe.configuration_ernie4_5_moe import Ernie4_5_MoeConfig
+        cfg = Ernie4_5_MoeConfig(hidden_size=hidden, moe_intermediate_size=inter, intermediate_size=inter,
+                                 moe_num_experts=E, moe_k=k, moe_num_shared_experts=2, hidden_act="silu",
+                                 use_bias=False)
+        router, forward = random_ernie_router(E, hidden, k, dev, dtype), hf.ernie4_5_moe_forward
+    return cfg, MOEParams(router, experts, E, k), forward
+
+
+@pytest.mark.parametrize("model", ["olmoe", "qwen3", "ernie"])
+def test_package_hf_reference_forward_functions_cpu(model):
+    """moe_explore.hf_moe_reference (the reference's hf_moe_reference.py:16-120) on the CPU in fp32
+    against the package's topk_moe_torch and against the oracle, on the same parameter record."""
+    from moe_explore.functional.topk_moe import topk_moe_torch
+    hidden, inter, E, k, T = 64, 32, 8, 2, 40
+    torch.manual_seed(3)
+    cfg, params, forward = _hf_case(model, hidden, inter, E, k, "cpu", torch.float32)
+    x = torch.randn((T, hidden))
+    ref = forward(cfg, x.unsqueeze(0), params).squeeze(0)
+    assert_parity(topk_moe_torch(x, params), ref, torch.float32, f"{model}: topk_moe_torch vs transformers")
+    ep = params.expert_params
+    want, _, _ = _oracle_layer(x, type(params)(params.router_params, type(ep)(
+        ep.gate_weight, ep.up_weight, ep.down_weight, "swiglu"), E, k))
+    assert_parity(ref, want, torch.float32, f"{model}: transformers vs oracle")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("model", ["olmoe", "qwen3", "ernie"])
+def test_package_hf_reference_forward_functions(model):
+    """The package's own counterpart of the reference's hf_moe_reference.py (its *_forward
+    functions on a config and a MOEParams record) against topk_moe_forward on the same record,
+    as the reference's tests/test_hf.py:75-99 does with released configs; here the configs are
+    built locally at a reduced size, bf16 on the GPU, the reference's comparison rule."""
+    from moe_explore.functional.topk_moe import topk_moe_forward
+    from moe_explore.testing import assert_close
+    hidden, inter, E, k, T = 256, 128, 16, 4, 200
+    dev, dtype = "cuda", torch.bfloat16
+    torch.manual_seed(11)
+    cfg, params, forward = _hf_case(model, hidden, inter, E, k, dev, dtype)
+    x = torch.randn((T, hidden), device=dev, dtype=dtype)
+    ref = forward(cfg, x.unsqueeze(0), params).squeeze(0)
+    out = topk_moe_forward(x, params)
+    assert ref.isfinite().all() and out.isfinite().all()
+    assert_close(ref, out)
