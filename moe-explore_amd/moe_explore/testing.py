@@ -36,6 +36,26 @@ def torch_grouped_matmul_gather_scatter(a, params):
     return c.to(dtype)
 
 
+def torch_grouped_glu(a, params):
+    """Grouped GLU with separate gate and up weights and an optional fused gather
+    (``testing.py:52-85``): ``c[rows of group i] = act(a_i @ gate[i]) * (a_i @ up[i])``.
+    ``params`` is any record with ``gate_weight``, ``up_weight`` ``[E, K, N]``,
+    ``group_indices`` ``[E + 1]``, ``permute_indices``, ``gather``, ``topk`` and ``activation``
+    ("silu" or "gelu", applied to the gate product)."""
+    assert params.gate_weight.size() == params.up_weight.size()
+    gather = bool(getattr(params, "gather", False))
+    topk = getattr(params, "topk", 1)
+    rows = params.permute_indices // topk if gather else None
+    c = torch.zeros((a.size(0) * topk if gather else a.size(0), params.gate_weight.size(-1)),
+                    device=a.device, dtype=a.dtype)
+    bounds = params.group_indices.tolist()
+    for i in range(params.gate_weight.size(0)):
+        lo, hi = bounds[i], bounds[i + 1]
+        a_i = a[rows[lo:hi]] if gather else a[lo:hi]
+        c[lo:hi] = activation(a_i @ params.gate_weight[i], params.activation) * (a_i @ params.up_weight[i])
+    return c
+
+
 def perfect_routing(num_tokens, num_experts, topk, device, dtype):
     """Every expert gets the same number of rows (``testing.py:87-95``)."""
     assert num_tokens % num_experts == 0

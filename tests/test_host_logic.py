@@ -132,3 +132,33 @@ def test_stage_ranges_are_off_by_default_and_nest():
     assert not tracing.enabled()
     with tracing.scope("router"):
         pass
+
+
+@pytest.mark.parametrize("gather", [False, True])
+def test_grouped_glu_helper_matches_the_interleaved_oracle(gather):
+    """testing.torch_grouped_glu (separate gate / up weights, testing.py:52-85) against the oracle's
+    grouped product on the interleaved weight with the GLU epilogue."""
+    from types import SimpleNamespace
+    from moe_explore.functional.activation import glu_form
+    from moe_explore.testing import torch_grouped_glu
+    from oracle import moe_ref
+    g = torch.Generator().manual_seed(9)
+    T, E, k, K, N = 37, 5, 2, 24, 16
+    gate = torch.randn((E, K, N), generator=g)
+    up = torch.randn((E, K, N), generator=g)
+    w = torch.stack((gate, up), dim=-1).reshape(E, K, 2 * N)
+    if gather:
+        idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+        gi, perm = moe_ref.get_token_indices(idx, k, E, zero_prefix=True)
+        a = torch.randn((T, K), generator=g)
+    else:
+        perm = None
+        gi = torch.tensor([0, 4, 4, 20, 30, 37], dtype=torch.int32)
+        a = torch.randn((37, K), generator=g)
+    for act in ("silu", "gelu"):
+        p = SimpleNamespace(gate_weight=gate, up_weight=up, group_indices=gi, permute_indices=perm,
+                            gather=gather, topk=k if gather else 1, activation=act)
+        got = torch_grouped_glu(a, p)
+        want = moe_ref.grouped_matmul_gather_scatter(a, w, gi, perm, gather=gather, topk=k if gather else 1,
+                                                     activation_name=glu_form(act))
+        torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-5)
