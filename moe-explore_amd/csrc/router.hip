@@ -98,7 +98,7 @@ __device__ __forceinline__ float4 load4_as_f32(const TX* p) {
 // NB: 32-expert blocks a wavefront accumulates.  EC: chunks of NB * 32 experts; with more
 // than one, wavefront w works on chunk w % EC and the wavefronts of a chunk split K (more
 // than 256 experts: NB = 8, EC = 2).  MBW: 32-token blocks of a workgroup (every weight
-// fragment is used MBW times; only 1 is instantiated).  U: K steps whose loads are issued
+// fragment is used MBW times; 2 for 129-256 experts and many tokens, else 1).  U: K steps whose loads are issued
 // together.  LPT: lanes that share a token in the selection phase (8, or 16 with eight
 // wavefronts and more than 64 experts, where the selection is most of the kernel).  Dynamic LDS: the logits of the workgroup's tokens, kBlock * MBW * (EC * NB * 32 + 1)
 // floats.
@@ -466,6 +466,18 @@ int launch_fwd(const RouterArgs& g, hipStream_t stream) {
   else if (nb <= 2) router_fwd_kernel<TX, F32, 2, 1, 8><<<grid, block, lds_bytes(64), stream>>>(g);
   else if (nb <= 4 && block.x == 512) router_fwd_kernel<TX, F32, 4, 1, 4, 1, 16><<<grid, block, lds_bytes(128), stream>>>(g);
   else if (nb <= 4) router_fwd_kernel<TX, F32, 4, 1, 4><<<grid, block, lds_bytes(128), stream>>>(g);
+  else if (nb <= 8 && wgs > num_cus()) {
+    // 129-256 experts and more 32-token blocks than compute units: 64 tokens a workgroup, two
+    // groups of four wavefronts with 128 experts each, so that every weight fragment (the
+    // 2 MiB weight is re-read from L2 by every workgroup) serves two token blocks
+    // (d = 4096, E = 256: T = 16384 220 -> 167 us, T = 32768 440 -> 335 us; with one round of
+    // workgroups or less the 32-token form is faster, 115 against 156 us at T = 8192)
+    auto kernel = router_fwd_kernel<TX, F32, 4, 2, 4, 2, 16>;
+    const size_t lds = 2 * lds_bytes(256);
+    const int rc = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lds);
+    if (rc != MOE_OK) return rc;
+    kernel<<<dim3(static_cast<unsigned>((g.T + 2 * kBlock - 1) / (2 * kBlock))), dim3(512), lds, stream>>>(g);
+  }
   else if (nb <= 8 && block.x == 512) router_fwd_kernel<TX, F32, 8, 1, 2, 1, 16><<<grid, block, lds_bytes(256), stream>>>(g);
   else if (nb <= 8) router_fwd_kernel<TX, F32, 8, 1, 2><<<grid, block, lds_bytes(256), stream>>>(g);
   else {

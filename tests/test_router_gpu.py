@@ -212,3 +212,15 @@ def test_unsupported_shapes_take_the_aten_path():
     s, i = topk_router(x.cuda(), TopkRouterParams(w.cuda(), 2, True, True))
     so, io = moe_ref.topk_router(x, w, 2, True, True)
     assert s.shape == so.shape and i.shape == io.shape
+
+
+@pytest.mark.parametrize("E,topk", [(256, 8), (160, 6)])
+def test_topk_router_many_tokens_and_129_to_256_experts(E, topk):
+    """More 32-token blocks than compute units and 129-256 experts: the kernel form with 64
+    tokens a workgroup (two groups of wavefronts, 128 experts each)."""
+    from moe_explore.params import TopkRouterParams
+    from moe_explore.router import topk_router
+    T, d = 32 * 300 + 17, 256
+    x, w = _inputs(T, d, E, torch.bfloat16, seed=E)
+    s, i = topk_router(x.cuda(), TopkRouterParams(w.cuda(), topk, True, True))
+    _check(s.cpu(), i.cpu(), x, w, topk, True, True)
