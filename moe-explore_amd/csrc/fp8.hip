@@ -144,11 +144,6 @@ __device__ __forceinline__ void wait_copies_keep_youngest_and_barrier() {
   asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(YOUNGEST) : "memory");
 }
 
-struct NextDraw {
-  unsigned* slot;   // queue word the next draw goes to (nullptr: every queue has run dry)
-  unsigned value;   // what the draw returned (thread 0)
-  bool drawn;
-};
 
 // One work item: `tpw` adjacent column tiles of one row block, computed as ONE stream of K
 // steps (token addresses stay, weight addresses move on), so that the copies of the next
@@ -528,7 +523,7 @@ __device__ __forceinline__ void fp8_work_item(const Fp8Args& fa, const Sched s, 
 }
 
 // One resident workgroup per compute unit draws work item ids from the tile queues of the
-// launch stream (gemm_mfma_dma.hip describes them: id 8j + q belongs to queue q, a workgroup
+// launch stream (gemm_mfma.h describes them: id 8j + q belongs to queue q, a workgroup
 // draws from the queue of its XCD first, word 8 counts the workgroups that are done and the
 // last one clears the set); without a queue set (a launch that is being captured) workgroup b
 // takes ids b, b + gridDim.x, ...
@@ -560,6 +555,8 @@ __global__ __launch_bounds__(kThreads) void m_grouped_fp8_kernel(Fp8KernelArgs k
       *sh_next = static_id < args->s.wgs ? static_cast<int>(static_id) : -1;
       static_id += gridDim.x;
     } else if (threadIdx.x == 0) {
+      // (draw_work_item() of gemm_mfma.h written out: called as a function this kernel measured 2 %
+      // slower at T = 1024 and 8192, the scalar registers of its K loop falling differently)
       unsigned* const queue = args->queue;
       const int total = static_cast<int>(args->s.wgs);
       int id = -1;

@@ -106,6 +106,63 @@ inline Sched make_sched(const MGemmArgs& g, int BM, int tpw = 1) {
   return s;
 }
 
+// ---- tile queues of the persistent kernels ---------------------------------------------
+// A launch has one resident workgroup per compute unit; every workgroup draws work item ids
+// until none is left.  Id 8 j + q belongs to queue q: a workgroup draws from the queue of the
+// XCD it runs on (its ids share the panels they stream, and an XCD has its own L2), then from
+// the other queues, so every id is drawn whatever XCDs the launch lands on.  A queue set is 16
+// words: eight draw counters, then the count of workgroups that are done; the last one clears
+// the set for the next launch that uses it (sets belong to one stream: gemm.h).
+struct NextDraw {
+  unsigned* slot;   // queue word the next draw goes to (nullptr: every queue has run dry)
+  unsigned value;   // what a draw made ahead of time returned (thread 0)
+  bool drawn;
+};
+
+// Thread 0: the next id of this workgroup, or -1.  `tried`: queues found dry so far, the home
+// queue first.  A draw made ahead of time (during the last store of the item before, so that the
+// atomic's round trip runs under the store) is in `next`.
+__device__ __forceinline__ int draw_work_item(unsigned* queue, int total, int home, int& tried,
+                                              NextDraw& next) {
+  int id = -1;
+  while (tried < kNumXcd) {
+    const int q = (home + tried) & (kNumXcd - 1);
+    const unsigned got = next.drawn ? next.value : atomicAdd(&queue[q], 1u);
+    next.drawn = false;
+    const int64_t cand = static_cast<int64_t>(got) * kNumXcd + q;
+    if (cand < total) {
+      id = static_cast<int>(cand);
+      break;
+    }
+    ++tried;
+    // A queue that has run dry stays dry for the rest of the launch: look at all the
+    // counters at once (one round trip) and pass over the dry ones, instead of finding
+    // each of them empty with an atomic of its own when the launch drains.
+    unsigned seen[kNumXcd];
+#pragma unroll
+    for (int i = 0; i < kNumXcd; ++i)
+      seen[i] = __hip_atomic_load(&queue[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while (tried < kNumXcd) {
+      const int qq = (home + tried) & (kNumXcd - 1);
+      unsigned c = 0;
+#pragma unroll
+      for (int i = 0; i < kNumXcd; ++i) c = i == qq ? seen[i] : c;
+      if (static_cast<int64_t>(c) * kNumXcd + qq < total) break;
+      ++tried;
+    }
+  }
+  next.slot = tried < kNumXcd ? &queue[(home + tried) & (kNumXcd - 1)] : nullptr;
+  return id;
+}
+
+// Thread 0 of a workgroup that has run out of work (each queue runs dry after total / 8 draws).
+__device__ __forceinline__ void leave_queues(unsigned* queue) {
+  __threadfence();
+  if (atomicAdd(&queue[kNumXcd], 1u) == gridDim.x - 1) {
+    for (int q = 0; q <= kNumXcd; ++q) atomicExch(&queue[q], 0u);
+  }
+}
+
 // Wavefront 0 finds the expert whose row blocks contain block `mt`.
 template <int BM>
 __device__ __forceinline__ void find_tile(const int32_t* __restrict__ gi, int E, int P, int mt,

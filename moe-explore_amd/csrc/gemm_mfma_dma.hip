@@ -85,11 +85,6 @@ __device__ __forceinline__ void wait_copies_keep_youngest_and_barrier() {
 // ACT: epilogue code, or kGluBwd + the GLU code for the fused GLU backward
 // (store_tile_glu_bwd16).
 constexpr int kGluBwd = 16;
-struct NextDraw {
-  unsigned* slot;   // queue word the next draw goes to (nullptr: every queue has run dry)
-  unsigned value;   // what the draw returned (thread 0)
-  bool drawn;
-};
 
 // `next`: thread 0 draws the id of the workgroup's next work item right before the last store
 // of this one, so that the atomic's round trip runs under the store instead of after it.
@@ -488,38 +483,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void m_grouped_dma_kernel(DmaKernel
       *sh_next = static_id < args->s.wgs ? static_cast<int>(static_id) : -1;
       static_id += gridDim.x;
     } else if (threadIdx.x == 0) {
-      unsigned* const queue = args->queue;
-      const int total = static_cast<int>(args->s.wgs);
-      int id = -1;
-      while (tried < kNumXcd) {
-        const int q = (home + tried) & (kNumXcd - 1);
-        // (a draw made during the last store went to this same queue)
-        const unsigned got = next.drawn ? next.value : atomicAdd(&queue[q], 1u);
-        next.drawn = false;
-        const int64_t cand = static_cast<int64_t>(got) * kNumXcd + q;
-        if (cand < total) {
-          id = static_cast<int>(cand);
-          break;
-        }
-        ++tried;
-        // A queue that has run dry stays dry for the rest of the launch: look at all the
-        // counters at once (one round trip) and pass over the dry ones, instead of finding
-        // each of them empty with an atomic of its own when the launch drains.
-        unsigned seen[kNumXcd];
-#pragma unroll
-        for (int i = 0; i < kNumXcd; ++i)
-          seen[i] = __hip_atomic_load(&queue[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        while (tried < kNumXcd) {
-          const int qq = (home + tried) & (kNumXcd - 1);
-          unsigned c = 0;
-#pragma unroll
-          for (int i = 0; i < kNumXcd; ++i) c = i == qq ? seen[i] : c;
-          if (static_cast<int64_t>(c) * kNumXcd + qq < total) break;
-          ++tried;
-        }
-      }
-      *sh_next = id;
-      next.slot = tried < kNumXcd ? &queue[(home + tried) & (kNumXcd - 1)] : nullptr;
+      *sh_next = draw_work_item(args->queue, static_cast<int>(args->s.wgs), home, tried, next);
     }
     __syncthreads();
     const int id = __builtin_amdgcn_readfirstlane(*sh_next);
@@ -527,13 +491,7 @@ __global__ __launch_bounds__(64 * WVM * WVN) void m_grouped_dma_kernel(DmaKernel
     m_grouped_dma_tile<T, BM, WVM, WVN, WL, ACT>(args->g, args->s, id, next);
   }
   // (every workgroup ends here: each queue runs dry after s.wgs / 8 draws)
-  if (threadIdx.x == 0 && ka.queue != nullptr) {
-    unsigned* const queue = ka.queue;
-    __threadfence();
-    if (atomicAdd(&queue[kNumXcd], 1u) == gridDim.x - 1) {
-      for (int q = 0; q <= kNumXcd; ++q) atomicExch(&queue[q], 0u);
-    }
-  }
+  if (threadIdx.x == 0 && ka.queue != nullptr) leave_queues(ka.queue);
 }
 
 // The queue set of `stream` on the current device and the number of compute units of that
