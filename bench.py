@@ -125,7 +125,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--mode", choices=["fwdbwd", "fwd"], default="fwdbwd")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23", "fp8", "digest", "ablation"],
+    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23", "models", "fp8", "digest", "ablation"],
                     default="all",
                     help="profiling aids: 'kernel' launches only the dominant GEMM --steps times, "
                          "'copy' only a 1 GiB device copy (the known-size kernel that calibrates "
@@ -135,7 +135,10 @@ def main():
                          "combine) at the shapes of configs 1-3 with their algorithmic bytes and "
                          "event-timed GB/s, 'configs23' the routed experts (forward, then forward + "
                          "backward) at the shapes of configs 2 and 3, config 3 with Zipf(1.2) expert "
-                         "loads, 'fp8' the fp8 inference layer (config 4: T = 128, 1024, 8192, GeGLU) "
+                         "loads, 'models' the whole layer (router included; forward, then forward + backward) "
+                         "at the Qwen3-30B-A3B, OLMoE-1B-7B and Ernie-4.5 layer shapes with 32000 tokens "
+                         "(the shapes and the token count of the reference's bench_glu.py / profile_proton.py), "
+                         "'fp8' the fp8 inference layer (config 4: T = 128, 1024, 8192, GeGLU) "
                          "with its weight-streaming rate and TFLOP/s, 'digest' prints the digest of "
                          "the dominant kernel's sources that a profile summary records, 'ablation' times "
                          "the four GEMM shapes of config 1 (gate/up, dX, G without its fused epilogue, "
@@ -348,6 +351,50 @@ def main():
                 print("%s T=%d d=%d ff=%d E=%d top-%d rows/expert %d..%d  %-8s %8.3f ms %7.1f TFLOP/s" % (
                     name, T, d, ff, E, k, cnt.min().item(), cnt.max().item(), label, ms,
                     units * R * d * ff / ms / 1e9), flush=True)
+        return
+    if args.only == "models":
+        # (bench/bench_glu.py:74-103 for the shapes, bench/profile_proton.py:16-21 for the tokens;
+        # under `rocprofv3 --kernel-trace --stats` the kernels are the stages of the reference's
+        # profile: router, get_token_indices, fused grouped GLU, down grouped GEMM, scale_and_reduce)
+        from moe_explore.params import ErnieRouterParams
+        for name, d, ff, E, k, ernie in (("Qwen3-30B-A3B", 2048, 768, 128, 8, False),
+                                         ("OLMoE-1B-7B", 2048, 1024, 64, 8, False),
+                                         ("Ernie-4.5-21B-A3B", 2560, 1536, 64, 6, True)):
+            torch.manual_seed(0)
+            T, dt = 32000, torch.bfloat16
+            R = T * k
+            x = torch.randn(T, d, device=dev, dtype=dt).requires_grad_(True)
+            w1 = (torch.randn(E, d, 2 * ff, device=dev, dtype=dt) * 0.02).requires_grad_(True)
+            w2 = (torch.randn(E, ff, d, device=dev, dtype=dt) * 0.02).requires_grad_(True)
+            if ernie:
+                wr = (torch.randn(d, E, device=dev) * d ** -0.5).requires_grad_(True)
+                rp = ErnieRouterParams(wr, torch.rand(E, device=dev) * (2.0 / E), k)
+            else:
+                wr = (torch.randn(d, E, device=dev, dtype=dt) * d ** -0.5).requires_grad_(True)
+                rp = TopkRouterParams(wr, k, softmax_before_topk=True, normalize_routing=True)
+            mp = MOEParams(rp, GLUInterleavedParams(w1, w2, "swiglu"), E, k)
+            dout = torch.randn(T, d, device=dev, dtype=dt)
+
+            def fwd():
+                with torch.no_grad():
+                    topk_moe_forward(x, mp)
+
+            def fwdbwd():
+                x.grad = w1.grad = w2.grad = wr.grad = None
+                topk_moe_forward(x, mp).backward(dout)
+
+            for fn, units, label in ((fwd, 6, "fwd"), (fwdbwd, 18, "fwd+bwd")):
+                for _ in range(args.warmup):
+                    fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    fn()
+                torch.cuda.synchronize()
+                ms = (time.perf_counter() - t0) / args.steps * 1e3
+                print("%-18s T=%d d=%d ff=%d E=%d top-%d  %-8s %8.3f ms %7.1f TFLOP/s" % (
+                    name, T, d, ff, E, k, label, ms, units * R * d * ff / ms / 1e9), flush=True)
+            del x, w1, w2, wr, dout, mp
         return
     T, d, ff, E, k = cfg["T"], cfg["d"], cfg["ff"], cfg["E"], cfg["k"]
     R = T * k

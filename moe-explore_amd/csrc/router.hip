@@ -464,6 +464,13 @@ int launch_fwd(const RouterArgs& g, hipStream_t stream) {
   auto lds_bytes = [](int experts) { return static_cast<size_t>(kBlock) * (experts + 1) * sizeof(float); };
   if (nb <= 1) router_fwd_kernel<TX, F32, 1, 1, 16><<<grid, block, lds_bytes(32), stream>>>(g);
   else if (nb <= 2) router_fwd_kernel<TX, F32, 2, 1, 8><<<grid, block, lds_bytes(64), stream>>>(g);
+  else if (nb <= 4 && block.x == 512 && wgs > num_cus()) {
+    // 65-128 experts, more than one round of 32-token workgroups (and fewer than the 2048 from
+    // which four wavefronts a workgroup do better): 64 tokens a workgroup, every weight fragment
+    // serving two token blocks (E = 128, d = 2048: T = 16384 88 -> 70 us, T = 32000 166 -> 133 us)
+    const dim3 grid2(static_cast<unsigned>((g.T + 2 * kBlock - 1) / (2 * kBlock)));
+    router_fwd_kernel<TX, F32, 4, 2, 4, 1, 16><<<grid2, block, 2 * lds_bytes(128), stream>>>(g);
+  }
   else if (nb <= 4 && block.x == 512) router_fwd_kernel<TX, F32, 4, 1, 4, 1, 16><<<grid, block, lds_bytes(128), stream>>>(g);
   else if (nb <= 4) router_fwd_kernel<TX, F32, 4, 1, 4><<<grid, block, lds_bytes(128), stream>>>(g);
   else if (nb <= 8 && wgs > num_cus()) {

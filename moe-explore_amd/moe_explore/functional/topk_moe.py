@@ -116,6 +116,10 @@ def _ksplit_for(rows, num_experts, n, k):
     return 1
 
 
+# intermediate width below which the dW2 kernel gathers its token rows itself (see backward)
+_FUSED_GATHER_BELOW_FF = 1280
+
+
 class _ExpertsFunction(torch.autograd.Function):
     """Routed experts + combine: ``out[t] = sum_j scores[t,j] * FFN_e(t,j)(x[t])``."""
 
@@ -171,11 +175,17 @@ class _ExpertsFunction(torch.autograd.Function):
         # over R x d each): the K-grouped kernel then reads that operand from LDS with plain
         # 16-byte loads instead of transpose loads (-10 % on dW1 at the Mixtral shape).  The
         # kernel can also gather by itself, but then has to wait for the row ids of every K
-        # step, and with them for the copies it keeps in flight: 10-15 % slower.
+        # step, and with them for the copies it keeps in flight: 10-15 % slower.  That is still
+        # the cheaper way for dW2 of narrow experts: the pass over R x d costs ~330 / ff of the
+        # GEMM it serves (ff = 1024: a third), so below ff = 1280 the kernel gathers dout itself
+        # (OLMoE shape, T = 8192: 0.362 -> 0.316 ms; Qwen3 shape, T = 32000: 1.09 -> 0.91 ms;
+        # ff = 1408 the same either way; dW1, whose GEMM is twice as long, gathers first).
         if ctx.needs_input_grad[2]:
-            dt = row_gather_kmajor(dout, idx, topk, gi)
+            dt = None if a_scaled.size(1) < _FUSED_GATHER_BELOW_FF else row_gather_kmajor(dout, idx, topk, gi)
             if dt is not None:
                 dw2 = k_grouped_gemm(a_scaled, dt, gi, b_kmajor=True)
+            elif a_scaled.size(1) < _FUSED_GATHER_BELOW_FF:
+                dw2 = k_grouped_gemm(a_scaled, dout, gi, idx, topk, gather_b=True)
             else:
                 dw2 = k_grouped_gemm(a_scaled, row_gather(dout, idx, topk), gi)
         if ctx.needs_input_grad[1]:

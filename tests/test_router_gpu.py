@@ -214,10 +214,10 @@ def test_unsupported_shapes_take_the_aten_path():
     assert s.shape == so.shape and i.shape == io.shape
 
 
-@pytest.mark.parametrize("E,topk", [(256, 8), (160, 6)])
-def test_topk_router_many_tokens_and_129_to_256_experts(E, topk):
-    """More 32-token blocks than compute units and 129-256 experts: the kernel form with 64
-    tokens a workgroup (two groups of wavefronts, 128 experts each)."""
+@pytest.mark.parametrize("E,topk", [(256, 8), (160, 6), (128, 8), (100, 4)])
+def test_topk_router_many_tokens_and_65_to_256_experts(E, topk):
+    """More 32-token blocks than compute units and 65-256 experts: the kernel forms with 64
+    tokens a workgroup (129-256 experts: two groups of wavefronts, 128 experts each)."""
     from moe_explore.params import TopkRouterParams
     from moe_explore.router import topk_router
     T, d = 32 * 300 + 17, 256
