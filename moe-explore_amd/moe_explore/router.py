@@ -2,9 +2,10 @@
 
 On the GPU ``topk_router`` and ``ernie_router`` run as one fused HIP kernel (logits,
 fp32 softmax, top-k, renormalisation, cast) with a second small kernel for the gradient
-of the scores with respect to the logits; the two skinny matmuls of the backward pass
-stay on ATen.  Shapes outside the kernel's reach (more than 512 experts, top-k above 16,
-rows that cannot be read 16 bytes at a time) and CPU tensors take the ATen formulation
+of the scores with respect to the logits; of the two skinny matmuls of the backward pass dx
+stays on ATen and the weight gradient runs on the K-grouped kernel from 8192 tokens on.
+Shapes outside the kernel's reach (more than 512 experts, top-k above 16, rows that cannot be
+read 16 bytes at a time) and CPU tensors take the ATen formulation
 below, which is the reference's own.
 """
 import torch
@@ -67,6 +68,34 @@ def _fused_forward(x, weight, bias, topk, flags, want_logits):
     return scores, idx, logits
 
 
+_token_group_bounds = {}
+
+
+def _router_weight_grad(x, dlogits, out_dtype):
+    """``x^T @ dlogits`` ([T, d]^T [T, E] -> [d, E]).  A reduction over many tokens into a small
+    matrix, which the library's GEMM runs on a few compute units (T = 32000, d = 2048, E = 128:
+    109 us).  From 8192 tokens on the tokens are cut into as many groups as fill the GPU and the
+    K-grouped weight-gradient kernel computes one partial product a group (55 us with the sum of
+    the partials; 16-bit operands only: its partials are rounded to 16 bits, 2e-3 relative)."""
+    T, d = x.shape
+    E = dlogits.size(1)
+    if (x.dtype in (torch.bfloat16, torch.float16) and dlogits.dtype == x.dtype and out_dtype == x.dtype
+            and T >= 8192 and d % 8 == 0 and E % 8 == 0 and x.stride(1) == 1 and x.stride(0) % 8 == 0):
+        from moe_explore.gpu_utils import get_gpu_sm_count
+        from moe_explore.hip_kernels.m_grouped_gemm import k_grouped_gemm
+        groups = max(1, min(T // 64, -(-get_gpu_sm_count(x.device) // -(-d // 256))))
+        key = (T, groups, x.device)
+        bounds = _token_group_bounds.get(key)
+        if bounds is None:
+            step = T // groups // 64 * 64
+            bounds = torch.tensor([i * step for i in range(groups)] + [T], dtype=torch.int32, device=x.device)
+            if len(_token_group_bounds) > 64:
+                _token_group_bounds.clear()
+            _token_group_bounds[key] = bounds
+        return k_grouped_gemm(x, dlogits, bounds).float().sum(0)
+    return x.to(out_dtype).t() @ dlogits
+
+
 class _FusedRouter(torch.autograd.Function):
     """scores, indices = router(x, weight); differentiable in x and weight through the
     scores (the selection itself has no gradient)."""
@@ -99,7 +128,7 @@ class _FusedRouter(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             dx = (dlogits @ weight.t().to(out_dtype)).to(x.dtype)
         if ctx.needs_input_grad[1]:
-            dw = (x.to(out_dtype).t() @ dlogits).to(weight.dtype)
+            dw = _router_weight_grad(x, dlogits, out_dtype).to(weight.dtype)
         return dx, dw, None, None, None
 
 

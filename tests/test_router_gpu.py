@@ -224,3 +224,24 @@ def test_topk_router_many_tokens_and_65_to_256_experts(E, topk):
     x, w = _inputs(T, d, E, torch.bfloat16, seed=E)
     s, i = topk_router(x.cuda(), TopkRouterParams(w.cuda(), topk, True, True))
     _check(s.cpu(), i.cpu(), x, w, topk, True, True)
+
+
+def test_router_weight_gradient_with_many_tokens():
+    """From 8192 tokens on the router's weight gradient is a sum of partial products over token
+    groups from the K-grouped kernel: against fp32 autograd with the same selection, at the bf16 bar."""
+    from moe_explore.params import TopkRouterParams
+    from moe_explore.router import topk_router
+    T, d, E, topk = 8192 + 77, 256, 64, 8
+    x, w = _inputs(T, d, E, torch.bfloat16, seed=31)
+    g = torch.randn((T, topk), generator=seeded(8)).to(torch.bfloat16)
+    xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    s, i = topk_router(xg, TopkRouterParams(wg, topk, True, True))
+    s.backward(g.cuda())
+    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    logits = xr @ wr
+    logits = logits + (logits.to(torch.bfloat16).float() - logits).detach()
+    sr = torch.gather(torch.softmax(logits, -1), 1, i.cpu())
+    sr = sr / sr.sum(-1, keepdim=True)
+    sr.backward(g.float())
+    assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= 2e-2
+    assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 2e-2
