@@ -125,7 +125,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--mode", choices=["fwdbwd", "fwd"], default="fwdbwd")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23", "models", "fp8", "digest", "ablation"],
+    ap.add_argument("--only", choices=["all", "kernel", "copy", "router", "passes", "configs23", "models", "fp32", "fp8", "digest", "ablation"],
                     default="all",
                     help="profiling aids: 'kernel' launches only the dominant GEMM --steps times, "
                          "'copy' only a 1 GiB device copy (the known-size kernel that calibrates "
@@ -138,6 +138,8 @@ def main():
                          "loads, 'models' the whole layer (router included; forward, then forward + backward) "
                          "at the Qwen3-30B-A3B, OLMoE-1B-7B and Ernie-4.5 layer shapes with 32000 tokens "
                          "(the shapes and the token count of the reference's bench_glu.py / profile_proton.py), "
+                         "'fp32' the layer in fp32 (exact products on 32x32x2 fp32 MFMAs; forward, then "
+                         "forward + backward) with T = 8192, d = 2048, ff = 4096, E = 8, top-2, "
                          "'fp8' the fp8 inference layer (config 4: T = 128, 1024, 8192, GeGLU) "
                          "with its weight-streaming rate and TFLOP/s, 'digest' prints the digest of "
                          "the dominant kernel's sources that a profile summary records, 'ablation' times "
@@ -224,6 +226,39 @@ def main():
                 timed(lambda: k_grouped_gemm(a, dt, p.group_indices, b_kmajor=True), 2.0 * R * d * ff,
                       "dW2 (K-grouped, b K-major)", kind)
             del w1, w2, x, dout, dh, a, out, xt, dt
+        return
+    if args.only == "fp32":
+        # (157.3 TFLOP/s is the device's fp32 matrix-core peak)
+        T, d, ff, E, k = 8192, 2048, 4096, 8, 2
+        torch.manual_seed(0)
+        x = torch.randn(T, d, device=dev).requires_grad_(True)
+        w1 = (torch.randn(E, d, 2 * ff, device=dev) * 0.02).requires_grad_(True)
+        w2 = (torch.randn(E, ff, d, device=dev) * 0.02).requires_grad_(True)
+        wr = (torch.randn(d, E, device=dev) * d ** -0.5).requires_grad_(True)
+        mp = MOEParams(TopkRouterParams(wr, k, softmax_before_topk=True, normalize_routing=True),
+                       GLUInterleavedParams(w1, w2, "swiglu"), E, k)
+        dout = torch.randn(T, d, device=dev)
+
+        def fwd():
+            with torch.no_grad():
+                topk_moe_forward(x, mp)
+
+        def fwdbwd():
+            x.grad = w1.grad = w2.grad = wr.grad = None
+            topk_moe_forward(x, mp).backward(dout)
+
+        for fn, units, label in ((fwd, 6, "fwd"), (fwdbwd, 18, "fwd+bwd")):
+            for _ in range(args.warmup):
+                fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                fn()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) / args.steps * 1e3
+            tf = units * T * k * d * ff / ms / 1e9
+            print("fp32 layer T=%d d=%d ff=%d E=%d top-%d  %-8s %8.3f ms %7.1f TFLOP/s (%.2f of 157.3)" % (
+                T, d, ff, E, k, label, ms, tf, tf / 157.3), flush=True)
         return
     if args.only == "fp8":
         from moe_explore.fp8 import Fp8MLPParams, quantize_expert_weights, routed_experts_fp8

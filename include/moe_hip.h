@@ -172,8 +172,9 @@ MOE_API int moe_cast_from_f32(const float* src, int64_t src_stride, void* dst, i
  *           part i stores its partial product to c + i * c_split_stride elements and
  *           the caller adds the parts (moe_scale_and_reduce does).  MFMA kernel only,
  *           no epilogue; MOE_ERR_UNSUPPORTED otherwise.  Pass 1 and 0 for no split.
- * Shapes the MFMA kernels do not cover (fp32; K, N or strides not multiples of 8;
- * unaligned pointers) run on a scalar-FMA kernel with the same semantics.
+ * fp32 runs on fp32 MFMAs (exact products) when K, N and the strides are multiples of 4 and
+ * the pointers 16-byte aligned.  Shapes the MFMA kernels do not cover (16-bit: K, N or strides
+ * not multiples of 8; unaligned pointers) run on a scalar-FMA kernel with the same semantics.
  */
 MOE_API int moe_m_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, const void* w,
                        int64_t ldw_e, int64_t ldw_k, int64_t ldw_n, void* c, int64_t c_rows,

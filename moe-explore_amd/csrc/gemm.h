@@ -58,6 +58,11 @@ bool m_grouped_mfma_supported(const MGemmArgs& g);
 int launch_m_grouped_mfma(const MGemmArgs& g, hipStream_t stream);
 bool m_grouped_mfma_dma_supported(const MGemmArgs& g);  // K % 64 == 0, 16-byte stores, < 4 GiB spans
 int launch_m_grouped_mfma_dma(const MGemmArgs& g, hipStream_t stream);
+// fp32 on the matrix cores (exact products): K, N and strides multiples of 4, 16-byte aligned
+bool m_grouped_f32_mfma_supported(const MGemmArgs& g);
+int launch_m_grouped_f32_mfma(const MGemmArgs& g, hipStream_t stream);
+bool k_grouped_f32_mfma_supported(const KGemmArgs& g);
+int launch_k_grouped_f32_mfma(const KGemmArgs& g, hipStream_t stream);
 bool k_grouped_mfma_supported(const KGemmArgs& g);
 int launch_k_grouped_mfma(const KGemmArgs& g, hipStream_t stream);
 // The tile-queue set of `stream` on the current device (16 words of a __device__ array that

@@ -76,6 +76,7 @@ extern "C" int moe_m_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
   if (copy_preact) g.flags &= ~MOE_GEMM_SAVE_PREACT;
   int rc;
   if (!force_scalar() && m_grouped_mfma_supported(g)) rc = launch_m_grouped_mfma(g, s);
+  else if (!force_scalar() && m_grouped_f32_mfma_supported(g)) rc = launch_m_grouped_f32_mfma(g, s);
   else rc = launch_m_grouped_generic(g, s);
   if (rc != MOE_OK || !copy_preact) return rc;
   const size_t esz = dtype_bytes(dtype);
@@ -164,6 +165,7 @@ extern "C" int moe_k_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
               E, Ka,     Nb,  topk, flags, dtype, P, FastDiv(static_cast<uint32_t>(topk))};
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (!force_scalar() && k_grouped_mfma_supported(g)) return launch_k_grouped_mfma(g, s);
+  if (!force_scalar() && k_grouped_f32_mfma_supported(g)) return launch_k_grouped_f32_mfma(g, s);
   if (ka || kb)
     return fail(MOE_ERR_UNSUPPORTED, "K-major operands need the MFMA kernel (16-bit dtype, widths and "
                                      "strides multiples of 8, 16-byte aligned pointers)");

@@ -65,6 +65,41 @@ def test_k_grouped_gemm_tile_pipeline(sizes, gather):
             assert (out[e] == 0).all()
 
 
+@pytest.mark.parametrize("sizes", [
+    [0, 1, 64, 65, 0, 130, 7, 0],
+    [1] * 12,
+    [32, 31, 33, 0, 300],                      # segment ends on and next to K-step boundaries
+    [5, 0, 700, 0, 3, 64, 0, 0, 1, 250, 17, 0, 0, 90, 2, 66],
+])
+@pytest.mark.parametrize("Ka,Nb", [(776, 2568), (132, 36)])
+@pytest.mark.parametrize("gather", [None, "a", "b"])
+def test_k_grouped_gemm_fp32_matrix_core_kernel(sizes, Ka, Nb, gather):
+    """fp32 with widths that are multiples of 4 runs on 32x32x2 fp32 MFMAs: 256- and 128-row
+    output tiles (by tile count), ragged tile edges, ragged and empty segments, fetched rows."""
+    from moe_explore.triton_kernels.m_grouped_gemm import k_grouped_gemm
+    g = seeded(sum(sizes) + len(sizes) + Ka)
+    E, rows, topk = len(sizes), sum(sizes), 2
+    gi = torch.zeros(E + 1, dtype=torch.int32)
+    gi[1:] = torch.cumsum(torch.tensor(sizes), 0)
+    perm = torch.randperm(rows, generator=g)
+    tokens = (rows + topk - 1) // topk
+    a = randn((tokens if gather == "a" else rows, Ka), g, torch.float32)
+    b = randn((tokens if gather == "b" else rows, Nb), g, torch.float32)
+    if gather is None:
+        out = k_grouped_gemm(a.cuda(), b.cuda(), gi.cuda())
+        ref = moe_ref.k_grouped_matmul(a, b, gi)
+    else:
+        out = k_grouped_gemm(a.cuda(), b.cuda(), gi.cuda(), perm.cuda(), topk,
+                             gather_a=gather == "a", gather_b=gather == "b")
+        ref = moe_ref.k_grouped_matmul(a, b, gi, perm, topk, gather == "a", gather == "b")
+    assert_parity(out, ref, torch.float32, "fp32 k_grouped_gemm")
+    for e, n in enumerate(sizes):
+        if n == 0:
+            assert (out[e] == 0).all()
+        else:
+            assert_parity(out[e], ref[e], torch.float32, f"expert {e}")
+
+
 def test_k_grouped_gemm_many_uneven_experts():
     """100 experts with Zipf-like loads: the kernel numbers its tiles by expert rank and deals
     the chunks by load; ranks 64 and up come from the second half of the ranking."""

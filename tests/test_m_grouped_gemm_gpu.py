@@ -184,6 +184,66 @@ def test_large_ragged_groups_every_epilogue(dtype, activation, transposed):
     assert_parity(out.cpu(), ref, dtype, f"{activation} transposed={transposed}")
 
 
+@pytest.mark.parametrize("sizes", [[1025, 0, 5, 785, 1000, 529], [130, 0, 3, 64, 257, 31]])
+@pytest.mark.parametrize("K,N", [(28, 36), (36, 520), (100, 264), (256, 512)])
+@pytest.mark.parametrize("activation", [None, "silu", "gelu", "approx_gelu", "swiglu", "geglu"])
+@pytest.mark.parametrize("transposed", [False, True])
+def test_fp32_matrix_core_kernel(sizes, K, N, activation, transposed):
+    """fp32 with K, N multiples of 4 runs on 32x32x2 fp32 MFMAs: both tile heights (rows an
+    expert above and below 256), both weight layouts, every epilogue, K of one partial step,
+    a step and a partial one, several steps with a tail and whole steps, column tiles that are
+    partly outside the matrix; empty, tiny and tile-straddling groups."""
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    dtype = torch.float32
+    rows, E = sum(sizes), len(sizes)
+    g = seeded(rows + K * 3 + N + (7 if transposed else 0))
+    gi = torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32)
+    x = randn((rows, K), g, dtype)
+    w = randn((E, N, K) if transposed else (E, K, N), g, dtype, 0.1)
+    out = m_grouped_gemm(x.cuda(), _params(w.cuda(), gi.cuda(), None, False, False, rows, 1,
+                                           activation=activation), transpose_weight=transposed)
+    ref = moe_ref.grouped_matmul_gather_scatter(x, w.transpose(1, 2) if transposed else w, gi,
+                                                activation_name=activation)
+    assert out.shape == ref.shape
+    assert_parity(out.cpu(), ref, dtype, f"fp32 K={K} N={N} {activation} transposed={transposed}")
+
+
+@pytest.mark.parametrize("num_tokens,num_experts,topk", [(300, 8, 2), (3000, 4, 2)])
+@pytest.mark.parametrize("activation", [None, "swiglu"])
+def test_fp32_matrix_core_kernel_gather_scatter_combine(num_tokens, num_experts, topk, activation):
+    """The fp32 MFMA kernel with the fused row gather and saved pre-activation, the row
+    scatter and the weighted scatter-add."""
+    from moe_explore.expert_permute import get_token_indices
+    from moe_explore.functional.scale_and_reduce import scale_and_reduce
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    dtype, K, N = torch.float32, 200, 104
+    g = seeded(num_tokens + 5)
+    x = randn((num_tokens, K), g, dtype)
+    w = randn((num_experts, K, N), g, dtype, 1.0 / math.sqrt(N))
+    scores, idx = _routing(num_tokens, num_experts, topk, g, dtype)
+    p = get_token_indices(idx.view(-1).cuda(), topk, num_experts, zero_prefix=True)
+    out, pre = m_grouped_gemm(
+        x.cuda(), _params(w.cuda(), p.group_indices, p.indices, True, False, num_tokens, topk,
+                          activation=activation), save_preact=True)
+    ref, ref_pre = moe_ref.grouped_matmul_gather_scatter(
+        x, w, p.group_indices, p.indices, gather=True, num_tokens=num_tokens, topk=topk,
+        activation_name=activation, return_preact=True)
+    assert_parity(out, ref, dtype, "fp32 gather")
+    assert_parity(pre, ref_pre, dtype, "fp32 gather pre-activation")
+
+    xs = randn((num_tokens * topk, K), g, dtype)
+    params = _params(w.cuda(), p.group_indices, p.indices, False, True, num_tokens, topk,
+                     scales=scores.cuda(), activation=activation)
+    ref = moe_ref.grouped_matmul_gather_scatter(
+        xs, w, p.group_indices, p.indices, scatter=True, num_tokens=num_tokens, topk=topk,
+        scales=scores, activation_name=activation)
+    fused = m_grouped_gemm(xs.cuda(), params, combine=True)
+    assert_parity(fused, ref, dtype, "fp32 scatter-add")
+    rows = m_grouped_gemm(xs.cuda(), params)
+    two_pass = scale_and_reduce(rows, params.scales, num_tokens, topk, rows.size(-1))
+    assert_parity(two_pass, ref, dtype, "fp32 scatter + combine")
+
+
 @pytest.mark.parametrize("K,N", [(64, 272), (128, 528), (192, 1040)])
 @pytest.mark.parametrize("activation", [None, "swiglu"])
 @pytest.mark.parametrize("transposed", [False, True])
