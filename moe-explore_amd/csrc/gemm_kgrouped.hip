@@ -4,7 +4,7 @@
 // gathered).  The reference is forward-only; this is the transpose-side product
 // that autograd takes of its per-expert matmuls (functional/topk_moe.py:88-92).
 //
-// A workgroup (8 wavefronts, 2 x 4) computes 256 x 256 tiles of out[e], walking the
+// A workgroup (8 wavefronts, 2 x 4 or 4 x 2) computes 256 x 256 tiles of out[e], walking the
 // expert's row segment 64 positions at a time.  Both operands are stored with
 // the contraction index as the row, so both LDS tiles are [64 positions][256
 // features] and both fragment kinds are read with the LDS transpose load
@@ -44,10 +44,8 @@ using namespace mfma;
 typedef __attribute__((address_space(3))) void lds_void;
 
 constexpr int KBM = 256, KBN = 256;  // out tile: KBM features of a x KBN features of b
-constexpr int KWM = KBM / WAVES_M;   // 128
 constexpr int TILE_BYTES = BK * 256 * 2;  // 32 KiB per operand per stage
 constexpr int KSTAGE_BYTES = 2 * TILE_BYTES;
-constexpr int EPI_ROW_BYTES = WN * 2 + 8;            // 64 columns + pad: conflict-free writes
 
 __device__ __attribute__((aligned(512))) char g_zero_page[512];
 
@@ -181,7 +179,6 @@ __device__ __forceinline__ int balance_chunks(char* smem, const int32_t* group_i
 // per tile, launch + first-copy latency + store would be paid every 16 steps.
 // Tiles of experts without rows are zero-filled by the copy cursor when it passes
 // them.
-constexpr int EPI32_WAVE_BYTES = 32 * EPI_ROW_BYTES;  // 32 rows of a wave tile at a time
 constexpr int SHORT_BASE = 0;                // two stages of the operand copied one step ahead
 constexpr int LONG_BASE = 2 * TILE_BYTES;    // three stages of the operand copied two steps ahead
 constexpr int KLDS_BYTES = 5 * TILE_BYTES;   // 160 KiB, the whole LDS of a CU
@@ -189,7 +186,11 @@ constexpr int KLDS_BYTES = 5 * TILE_BYTES;   // 160 KiB, the whole LDS of a CU
 typedef const __attribute__((address_space(4))) int32_t* const_i32p;
 
 // KM: 0 = both operands position-major; 1 = a is K-major; 2 = b is K-major (then no gather).
-template <typename T, bool GA, bool GB, int KM>
+// WA: wavefronts along the a features, 2 (wave tiles of 128 a x 64 b features) or 4 (64 x 128).
+// The K-major operand is the wide side of the wave tile: eight of a wavefront's twelve fragments
+// per K half are then plain 16-byte reads and four are transpose-load pairs, for dW2 (b K-major)
+// as for dW1 (a K-major).
+template <typename T, bool GA, bool GB, int KM, int WA = 2>
 __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArgs g, KSched s,
                                                                         int ntiles) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -212,8 +213,10 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
   __syncthreads();  // the lists are read; from here on the LDS belongs to the copy pipeline
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm0 = (wave / WAVES_N) * KWM, wn0 = (wave % WAVES_N) * WN;
-
+  static_assert(WA == 2 || WA == 4, "2 x 4 or 4 x 2 wavefronts");
+  constexpr int WB = 8 / WA;
+  constexpr int WTM = KBM / WA, WTN = KBN / WB;  // wave tile: a features x b features
+  const int wm0 = (wave / WB) * WTM, wn0 = (wave % WB) * WTN;
 
   struct Tile {
     int e, mt, nt, lo, hi, KT;
@@ -402,11 +405,12 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
   };
 
   // ---- fragment reads ----------------------------------------------------------------------
-  // 16 x 16 x 32 MFMAs: the wavefront's 128 x 64 tile is 8 x 4 blocks of 16 x 16.  A K step is
-  // four units of 16 MFMAs: unit u = K half (u >> 1), half of the a blocks (u & 1); the b
-  // fragments of a K half serve both of its units.  Every fragment is two transpose loads:
-  // the 16-lane group lg fetches k rows 8*lg + i and + 4 of a 16-column block.
-  constexpr int MB16 = KWM / 16, NB16 = WN / 16, HB = MB16 / 2;
+  // 16 x 16 x 32 MFMAs: the wavefront's 128 x 64 (64 x 128) tile is 8 x 4 (4 x 8) blocks of
+  // 16 x 16.  A K step is four units of 16 MFMAs: unit u = K half (u >> 1), half of the a
+  // blocks (u & 1); the b fragments of a K half serve both of its units.  A fragment of a
+  // position-major tile is two transpose loads: the 16-lane group lg fetches k rows 8*lg + i
+  // and + 4 of a 16-column block.
+  constexpr int MB16 = WTM / 16, NB16 = WTN / 16, HB = MB16 / 2, NH = NB16 / 2;
   const int l16 = lane & 15, lg = lane >> 4;
   const int tr_i = (lane >> 2) & 3, tr_q = lane & 3;
   const int tr_c = 4 * tr_q;
@@ -429,11 +433,11 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
       else af[mb] = read_tr(at, u >> 1, wm0 + ((u & 1) * HB + mb) * 16);
     }
   };
-  // b blocks [2*half, 2*half + 2) of K half kh
+  // b blocks [NH*half, NH*half + NH) of K half kh
   auto read_unit_b = [&](int sstage, int lstage, int kh, int half, s16x8 (&bf)[NB16]) __attribute__((always_inline)) {
     const char* bt = A_SHORT ? smem + LONG_BASE + lstage * TILE_BYTES : smem + SHORT_BASE + sstage * TILE_BYTES;
 #pragma unroll
-    for (int nb = 2 * half; nb < 2 * half + 2; ++nb) {
+    for (int nb = NH * half; nb < NH * half + NH; ++nb) {
       if constexpr (KM == 2) bf[nb] = read_km(bt, kh, wn0 + nb * 16);
       else bf[nb] = read_tr(bt, kh, wn0 + nb * 16);
     }
@@ -446,9 +450,9 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
       for (int nb = 0; nb < NB16; ++nb) acc[mb][nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   };
   // b features as the first MFMA operand, a features as the second: a lane then owns one
-  // out row (an a feature) and four consecutive out columns (b features) per block.  Column
-  // blocks 0 and 1 come first: the fragments of blocks 2 and 3 are read at the start of the
-  // unit that first needs them, so that every unit reads the same 6 KiB.
+  // out row (an a feature) and four consecutive out columns (b features) per block.  The first
+  // half of the column blocks comes first: the fragments of the second half are read at the
+  // start of the unit that first needs them, so that every unit reads the same 6 KiB.
   auto multiply_unit = [&](int rh, s16x8 (&af)[HB], s16x8 (&bf)[NB16]) __attribute__((always_inline)) {
 #pragma unroll
     for (int nb = 0; nb < NB16; ++nb)
@@ -466,30 +470,35 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  // accumulators -> out tile of `t`, 32 rows of every wave tile at a time through `epi`
+  // accumulators -> out tile of `t`, PR rows of every wave tile at a time through `epi`
+  // (rows of WTN columns + pad: conflict-free writes)
+  constexpr int EPI_ROW_BYTES = WTN * 2 + 8;
+  constexpr int PR = WTN == 64 ? 32 : 16;
+  constexpr int EPI_WAVE_BYTES = PR * EPI_ROW_BYTES;
+  constexpr int ROW_LANES = WTN / 8;  // lanes that store one row piece, 16 bytes each
   auto store_acc = [&](const Tile& t, char* epi) __attribute__((always_inline)) {
     T* out = static_cast<T*>(g.out) + static_cast<int64_t>(t.e) * g.Ka * g.Nb;
     const int64_t m0 = static_cast<int64_t>(t.mt) * KBM, n0 = static_cast<int64_t>(t.nt) * KBN;
-    const int64_t col = n0 + wn0 + (lane & 7) * 8;
+    const int64_t col = n0 + wn0 + (lane % ROW_LANES) * 8;
 #pragma unroll
-    for (int pass = 0; pass < MB16 / 2; ++pass) {
+    for (int pass = 0; pass < WTM / PR; ++pass) {
 #pragma unroll
-      for (int mbh = 0; mbh < 2; ++mbh)
+      for (int mbh = 0; mbh < PR / 16; ++mbh)
 #pragma unroll
         for (int nb = 0; nb < NB16; ++nb) {
           T v[4];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) v[j] = from_f32<T>(acc[pass * 2 + mbh][nb][j]);
+          for (int j = 0; j < 4; ++j) v[j] = from_f32<T>(acc[pass * (PR / 16) + mbh][nb][j]);
           *reinterpret_cast<uint2*>(epi + (mbh * 16 + l16) * EPI_ROW_BYTES + (nb * 16 + lg * 4) * 2) =
               *reinterpret_cast<const uint2*>(v);
         }
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int r = it * 8 + (lane >> 3);
-        const char* src = epi + r * EPI_ROW_BYTES + (lane & 7) * 16;
+      for (int it = 0; it < PR * ROW_LANES / 64; ++it) {
+        const int r = it * (64 / ROW_LANES) + lane / ROW_LANES;
+        const char* src = epi + r * EPI_ROW_BYTES + (lane % ROW_LANES) * 16;
         uint2 v0 = *reinterpret_cast<const uint2*>(src);
         uint2 v1 = *reinterpret_cast<const uint2*>(src + 8);
-        const int64_t row = m0 + wm0 + pass * 32 + r;
+        const int64_t row = m0 + wm0 + pass * PR + r;
         if (row < g.Ka && col < g.Nb)
           *reinterpret_cast<uint4*>(out + row * g.Nb + col) = make_uint4(v0.x, v0.y, v1.x, v1.y);
       }
@@ -574,8 +583,8 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
     // their rows in the short one, 4-7 in the long one.
     if (!more) __syncthreads();
     const int lprev = lstage == 0 ? 2 : lstage - 1;
-    char* epi = wave < 4 ? smem + SHORT_BASE + (sstage ^ 1) * TILE_BYTES + wave * EPI32_WAVE_BYTES
-                         : smem + LONG_BASE + lprev * TILE_BYTES + (wave - 4) * EPI32_WAVE_BYTES;
+    char* epi = wave < 4 ? smem + SHORT_BASE + (sstage ^ 1) * TILE_BYTES + wave * EPI_WAVE_BYTES
+                         : smem + LONG_BASE + lprev * TILE_BYTES + (wave - 4) * EPI_WAVE_BYTES;
     store_acc(tc, epi);
     if (more) __syncthreads();  // later steps copy into the stages just used for the store
   }
@@ -684,13 +693,13 @@ int launch_k_grouped_mfma(const KGemmArgs& g, hipStream_t stream) {
   int rc;
   if (g.dtype == MOE_DTYPE_BF16) {
     if (km == 1) rc = launch(k_grouped_persistent_kernel<bf16_t, false, false, 1>);
-    else if (km == 2) rc = launch(k_grouped_persistent_kernel<bf16_t, false, false, 2>);
+    else if (km == 2) rc = launch(k_grouped_persistent_kernel<bf16_t, false, false, 2, 4>);
     else rc = ga ? launch(k_grouped_persistent_kernel<bf16_t, true, false, 0>)
                  : (gb ? launch(k_grouped_persistent_kernel<bf16_t, false, true, 0>)
                        : launch(k_grouped_persistent_kernel<bf16_t, false, false, 0>));
   } else {
     if (km == 1) rc = launch(k_grouped_persistent_kernel<f16_t, false, false, 1>);
-    else if (km == 2) rc = launch(k_grouped_persistent_kernel<f16_t, false, false, 2>);
+    else if (km == 2) rc = launch(k_grouped_persistent_kernel<f16_t, false, false, 2, 4>);
     else rc = ga ? launch(k_grouped_persistent_kernel<f16_t, true, false, 0>)
                  : (gb ? launch(k_grouped_persistent_kernel<f16_t, false, true, 0>)
                        : launch(k_grouped_persistent_kernel<f16_t, false, false, 0>));
