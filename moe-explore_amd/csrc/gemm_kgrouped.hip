@@ -594,15 +594,22 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
 // Gathers token rows into the K-major operand layout of the weight-gradient kernel:
 //     dst[f, qs(e) + (p - lo(e))] = src[idx[p] / div, f]      p in [lo(e), hi(e))
 // with qs(e) = 64 * (lo(e) / 64 + e), and zeros from the end of the expert's segment up to the
-// next multiple of 64 columns.  A workgroup moves 64 positions x 64 features through LDS:
-// 128-byte row pieces in (gathered rows of src), 128-byte row pieces out (feature rows of dst).
+// next multiple of 64 columns.  A workgroup moves 64 positions x 256 features through LDS, 64 x 64
+// at a time: 128-byte row pieces in (gathered rows of src), 128-byte row pieces out (feature rows
+// of dst).  The expert lookup and the row ids are paid once for the four feature blocks and
+// all their loads are in flight together: with one 64 x 64 block a workgroup the launch was
+// bound by that latency chain, not by memory.
+constexpr int kGatherFB = 4;  // 64-feature blocks a workgroup
 template <typename T>
 __global__ __launch_bounds__(256) void row_gather_kmajor_kernel(
     const T* __restrict__ src, int64_t src_rows, int64_t src_stride, const void* __restrict__ idx,
     int idx_bytes, FastDiv by_div, const int32_t* __restrict__ gi, int E, int P,
     T* __restrict__ dst, int64_t ld_dst, int64_t features) {
   __shared__ int sh[3];
-  __shared__ __attribute__((aligned(16))) T tile[64][64 + 8];
+  // (rows of 64 + 12 elements and eight-position groups in the transposing reads below: the four
+  // groups of a wavefront then read different banks; with 64 + 8 and sixteen-position groups
+  // every 2-byte read was a four-way bank conflict and the launch was bound by them)
+  __shared__ __attribute__((aligned(16))) T tile[kGatherFB][64][64 + 12];
   if (threadIdx.x < 64) find_tile<64>(gi, E, P, static_cast<int>(blockIdx.x), sh);
   __syncthreads();
   const int e = sh[0];
@@ -611,33 +618,45 @@ __global__ __launch_bounds__(256) void row_gather_kmajor_kernel(
   int lo = gi[e];
   lo = lo < 0 ? 0 : lo;
   const int64_t col0 = 64 * static_cast<int64_t>((lo >> 6) + e) + (row0 - lo);
-  const int64_t f0 = static_cast<int64_t>(blockIdx.y) * 64;
+  const int64_t f0 = static_cast<int64_t>(blockIdx.y) * (64 * kGatherFB);
   const int t = threadIdx.x;
-  {  // in: position t / 4, features 16 * (t % 4) .. +15
+  {  // in: position t / 4, features 16 * (t % 4) .. +15 of every block
     const int pos = t >> 2;
     const int p = row0 + pos;
     int64_t srow = 0;
     if (p < end) srow = clamp_index(by_div.div(load_index32(idx, idx_bytes, p)), src_rows);
+    uint4 v[kGatherFB][2];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int c = (t & 3) * 16 + h * 8;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (p < end && f0 + c < features)
-        v = *reinterpret_cast<const uint4*>(src + srow * src_stride + f0 + c);
-      *reinterpret_cast<uint4*>(&tile[pos][c]) = v;
-    }
-  }
-  __syncthreads();
-  {  // out: feature t / 4, positions 16 * (t % 4) .. +15
-    const int f = t >> 2;
-    if (f0 + f < features) {
+    for (int fb = 0; fb < kGatherFB; ++fb)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const int q = (t & 3) * 16 + h * 8;
+        const int64_t c = f0 + fb * 64 + (t & 3) * 16 + h * 8;
+        v[fb][h] = make_uint4(0, 0, 0, 0);
+        if (p < end && c < features) v[fb][h] = *reinterpret_cast<const uint4*>(src + srow * src_stride + c);
+      }
+#pragma unroll
+    for (int fb = 0; fb < kGatherFB; ++fb)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        uint2* dst2 = reinterpret_cast<uint2*>(&tile[fb][pos][(t & 3) * 16 + h * 8]);  // 8-byte aligned rows
+        dst2[0] = make_uint2(v[fb][h].x, v[fb][h].y);
+        dst2[1] = make_uint2(v[fb][h].z, v[fb][h].w);
+      }
+  }
+  __syncthreads();
+  {  // out: feature t / 4 of every block, positions 8 * (t % 4) .. +7 and 32 + those
+    const int f = t >> 2;
+#pragma unroll
+    for (int fb = 0; fb < kGatherFB; ++fb) {
+      const int64_t row = f0 + fb * 64 + f;
+      if (row >= features) continue;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int q = (t & 3) * 8 + h * 32;
         T v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = tile[q + j][f];
-        *reinterpret_cast<uint4*>(dst + (f0 + f) * ld_dst + col0 + q) = *reinterpret_cast<const uint4*>(v);
+        for (int j = 0; j < 8; ++j) v[j] = tile[fb][q + j][f];
+        *reinterpret_cast<uint4*>(dst + row * ld_dst + col0 + q) = *reinterpret_cast<const uint4*>(v);
       }
     }
   }
@@ -713,8 +732,9 @@ int launch_row_gather_kmajor(const void* src, int64_t src_rows, int64_t src_stri
                              int64_t P, void* dst, int64_t ld_dst, int64_t features, int dtype,
                              hipStream_t stream) {
   const int64_t blocks = P / 64 + E;  // static bound on the 64-position blocks of all experts
-  if (blocks > 0x7fffffff || (features + 63) / 64 > 65535) return fail(MOE_ERR_UNSUPPORTED, "grid too large");
-  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>((features + 63) / 64));
+  const int64_t fgroups = (features + 64 * kGatherFB - 1) / (64 * kGatherFB);
+  if (blocks > 0x7fffffff || fgroups > 65535) return fail(MOE_ERR_UNSUPPORTED, "grid too large");
+  const dim3 grid(static_cast<unsigned>(blocks), static_cast<unsigned>(fgroups));
   const FastDiv by_div(static_cast<uint32_t>(idx_div));
   if (dtype == MOE_DTYPE_BF16)
     row_gather_kmajor_kernel<bf16_t><<<grid, 256, 0, stream>>>(

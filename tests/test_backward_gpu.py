@@ -150,6 +150,8 @@ def test_k_grouped_gemm_more_experts_than_the_balanced_deal_takes(E, Ka, Nb):
     ([1000, 1030, 990, 1076], 2048, 256, torch.bfloat16),
     ([5] * 20, 77, 136, torch.float16),
     ([0, 0, 700], 350, 64, torch.bfloat16),
+    ([130, 0, 64, 1, 63, 65, 300, 0], 400, 328, torch.bfloat16),   # one feature group and a partial one
+    ([900, 1100], 1000, 1024, torch.float16),
 ])
 def test_row_gather_kmajor_layout(sizes, T, d, dtype):
     """moe_row_gather_kmajor: expert e's rows, transposed, start at column 64 * (lo // 64 + e)
