@@ -482,6 +482,7 @@ int launch_m_grouped_f32_mfma(const MGemmArgs& g, hipStream_t stream) {
   // 256-row blocks when groups are large, unless 128-row blocks fill the device's rounds of
   // workgroups markedly better (rounds x rows a block is the time of the launch)
   const int64_t nt = (g.N + BN - 1) / BN, cus = num_cus();
+  if (cus <= 0) return MOE_ERR_HIP;
   const int64_t cost256 = (((g.P + 255) / 256 + g.E) * nt + cus - 1) / cus * 256;
   const int64_t cost128 = (((g.P + 127) / 128 + g.E) * nt + cus - 1) / cus * 128;
   const bool big = g.P / g.E >= 256 && 10 * cost128 >= 9 * cost256;
@@ -499,7 +500,9 @@ bool k_grouped_f32_mfma_supported(const KGemmArgs& g) {
 int launch_k_grouped_f32_mfma(const KGemmArgs& g, hipStream_t stream) {
   // 256 x 256 tiles when they fill the device, else 128 x 256
   const int64_t tiles256 = ((g.Ka + 255) / 256) * ((g.Nb + BN - 1) / BN) * g.E;
-  return tiles256 >= num_cus() ? launch_k<256>(g, stream) : launch_k<128>(g, stream);
+  const int cus = num_cus();
+  if (cus <= 0) return MOE_ERR_HIP;
+  return tiles256 >= cus ? launch_k<256>(g, stream) : launch_k<128>(g, stream);
 }
 
 }  // namespace moe
