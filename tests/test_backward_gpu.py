@@ -330,6 +330,9 @@ def test_fused_glu_backward_declines_what_it_cannot_run():
     (64, 32, 48, 4, 2, "swiglu", torch.float32),
     (300, 128, 96, 8, 2, "geglu", torch.float32),
     (257, 64, 80, 8, 3, "silu", torch.float32),
+    # fp32 on the matrix cores with 256-row tiles (512 rows an expert) and every K-step path
+    (2048, 512, 768, 8, 2, "swiglu", torch.float32),
+    (1500, 260, 132, 4, 2, "geglu", torch.float32),
     (512, 256, 512, 8, 2, "swiglu", torch.bfloat16),
     (999, 256, 128, 64, 8, "swiglu", torch.bfloat16),
     (640, 128, 256, 8, 2, "gelu", torch.float16),
