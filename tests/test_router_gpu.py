@@ -245,3 +245,25 @@ def test_router_weight_gradient_with_many_tokens():
     sr.backward(g.float())
     assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= 2e-2
     assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 2e-2
+
+
+def test_ernie_router_gradients_with_many_tokens():
+    """fp32 router weight under bf16 activations, 8192 tokens and more: the backward products run
+    on 16-bit operands (dx) and over token groups on the K-grouped kernel (dW, returned in
+    fp32); against fp32 autograd with the same selection, at the bf16 bar."""
+    from moe_explore.params import ErnieRouterParams
+    from moe_explore.router import ernie_router
+    T, d, E, topk = 8192 + 33, 256, 64, 6
+    x, w = _inputs(T, d, E, torch.bfloat16, seed=41, w_dtype=torch.float32)
+    bias = torch.randn(E, generator=seeded(9)) * 0.05
+    g = torch.randn((T, topk), generator=seeded(10)).to(torch.bfloat16)
+    xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
+    s, i = ernie_router(xg, ErnieRouterParams(wg, bias.cuda(), topk))
+    s.backward(g.cuda())
+    assert wg.grad.dtype == torch.float32 and xg.grad.dtype == torch.bfloat16
+    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    sr = torch.gather(torch.softmax(xr @ wr, -1), 1, i.cpu())
+    sr = sr / sr.sum(-1, keepdim=True).clamp_min(1e-12)
+    sr.backward(g.float())
+    assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= 2e-2
+    assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 2e-2
