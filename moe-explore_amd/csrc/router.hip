@@ -446,6 +446,95 @@ __global__ __launch_bounds__(256) void router_bwd_kernel(const float* __restrict
   }
 }
 
+// The same gradient for up to 8 * EL experts (EL = 8 or 16), softmax before the top-k: a lane keeps its
+// EL logits and then its probabilities in registers (the general kernel reads the row three times and
+// calls expf three times an element), and the gradients of the selected scores reach their experts
+// through a row of LDS instead of a compare per (element, selected entry).
+template <typename TG, typename TO, int EL>
+__global__ __launch_bounds__(256) void router_bwd_small_kernel(const float* __restrict__ logits,
+                                                               const int64_t* __restrict__ idx,
+                                                               const TG* __restrict__ dscores,
+                                                               TO* __restrict__ dlogits, int64_t T, int E,
+                                                               int topk, int flags) {
+  constexpr int TB = 256 / kLpt;  // tokens a workgroup
+  __shared__ float dy_s[TB][EL * kLpt + 1];
+  const int tt = threadIdx.x / kLpt, q = threadIdx.x % kLpt;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * TB + tt;
+  if (t >= T) return;  // whole groups of kLpt lanes leave together; no workgroup barrier below
+  const bool ernie = flags & MOE_ROUTER_ERNIE;
+  const bool normalize = ernie || (flags & MOE_ROUTER_NORMALIZE);
+  const float* row = logits + t * E;
+  auto group_sum = [&](float v) __attribute__((always_inline)) {
+#pragma unroll
+    for (int o = 1; o < kLpt; o <<= 1) v += __shfl_xor(v, o, 64);
+    return v;
+  };
+  auto group_max = [&](float v) __attribute__((always_inline)) {
+#pragma unroll
+    for (int o = 1; o < kLpt; o <<= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+  };
+  float p[EL];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < EL; ++i) {
+    const int e = q + kLpt * i;
+    p[i] = e < E ? row[e] : -INFINITY;
+    mx = fmaxf(mx, p[i]);
+    dy_s[tt][e] = 0.0f;
+  }
+  mx = group_max(mx);
+  float z = 0.0f;
+#pragma unroll
+  for (int i = 0; i < EL; ++i) {
+    p[i] = q + kLpt * i < E ? expf(p[i] - mx) : 0.0f;
+    z += p[i];
+  }
+  z = group_sum(z);
+  const float rz = 1.0f / z;
+#pragma unroll
+  for (int i = 0; i < EL; ++i) p[i] *= rz;
+  // selected entries: lane q holds entries q and q + kLpt (topk <= 16)
+  int sel[2];
+  float raw[2], gs[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int j = q + kLpt * h;
+    sel[h] = -1;
+    raw[h] = 0.0f;
+    gs[h] = 0.0f;
+    if (j < topk) {
+      int e = static_cast<int>(idx[t * topk + j]);
+      e = e < 0 ? 0 : (e >= E ? E - 1 : e);
+      sel[h] = e;
+      gs[h] = to_f32(dscores[t * topk + j]);
+      raw[h] = expf(row[e] - mx) * rz;
+    }
+  }
+  // through the renormalisation: out_j = raw_j / S  ->  draw_j = (g_j - sum_l g_l out_l) / S
+  if (normalize) {
+    const float sum = group_sum(raw[0] + raw[1]);
+    const bool clamped = ernie && sum < 1e-12f;
+    const float S = clamped ? 1e-12f : sum;
+    float dot = group_sum((gs[0] * raw[0] + gs[1] * raw[1]) / S);
+    if (clamped) dot = 0.0f;  // the clamp passes no gradient to the sum
+    gs[0] = sel[0] >= 0 ? (gs[0] - dot) / S : 0.0f;
+    gs[1] = sel[1] >= 0 ? (gs[1] - dot) / S : 0.0f;
+  }
+  // through the softmax: dlogit_e = y_e (dy_e - sum_l dy_l y_l), y the softmax output
+  const float c = group_sum(gs[0] * raw[0] + gs[1] * raw[1]);
+  // (the lanes of a token sit in one wavefront: the zeros above are in place; the selected
+  // experts of a token are distinct)
+  if (sel[0] >= 0) dy_s[tt][sel[0]] = gs[0];
+  if (sel[1] >= 0) dy_s[tt][sel[1]] = gs[1];
+  TO* out = dlogits + t * E;
+#pragma unroll
+  for (int i = 0; i < EL; ++i) {
+    const int e = q + kLpt * i;
+    if (e < E) out[e] = from_f32<TO>(p[i] * (dy_s[tt][e] - c));
+  }
+}
+
 int64_t padded_k(int64_t d, bool f32) {
   const int64_t step = f32 ? 8 : 16;
   return (d + step - 1) / step * step;
@@ -585,6 +674,20 @@ int moe_router_bwd(const float* logits, const int64_t* topk_indices, const void*
   if (T == 0) return MOE_OK;
   MOE_REQUIRE(logits && topk_indices && dscores && dlogits, "router_bwd: null pointer");
   const dim3 grid(static_cast<unsigned>((T + 256 / kLpt - 1) / (256 / kLpt)));
+  const bool softmax_first = flags & (MOE_ROUTER_ERNIE | MOE_ROUTER_SOFTMAX_FIRST);
+  if (softmax_first && E <= 16 * kLpt) {
+    MOE_DISPATCH_DTYPE(g_dtype, TG, {
+      MOE_DISPATCH_DTYPE(out_dtype, TO, {
+        if (E <= 8 * kLpt)
+          router_bwd_small_kernel<TG, TO, 8><<<grid, 256, 0, stream>>>(
+              logits, topk_indices, static_cast<const TG*>(dscores), static_cast<TO*>(dlogits), T, E, topk, flags);
+        else
+          router_bwd_small_kernel<TG, TO, 16><<<grid, 256, 0, stream>>>(
+              logits, topk_indices, static_cast<const TG*>(dscores), static_cast<TO*>(dlogits), T, E, topk, flags);
+      });
+    });
+    return check_launch("router_bwd");
+  }
   MOE_DISPATCH_DTYPE(g_dtype, TG, {
     MOE_DISPATCH_DTYPE(out_dtype, TO, router_bwd_kernel<TG, TO><<<grid, 256, 0, stream>>>(
         logits, topk_indices, static_cast<const TG*>(dscores), static_cast<TO*>(dlogits), T, E, topk,
