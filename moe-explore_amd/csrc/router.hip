@@ -244,70 +244,141 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
     return v;
   };
 
-  // the reference's logits are a matmul result in the dtype of x (router.py:22); the
-  // Ernie router keeps them in fp32 (:44)
-  float mx = -INFINITY;
-  for (int e = q; e < E; e += LPT) {
-    float v = row[e];
-    if (!ernie && sizeof(TX) == 2) v = to_f32(from_f32<TX>(v));
-    row[e] = v;
-    if (g.logits_out != nullptr && t < g.T) g.logits_out[t * E + e] = v;
-    mx = fmaxf(mx, v);
-  }
-  mx = group_max(mx);
-  if (softmax_first) {
-    float z = 0.0f;
-    for (int e = q; e < E; e += LPT) {
-      const float p = expf(row[e] - mx);
-      row[e] = p;
-      z += p;
-    }
-    z = group_sum(z);
-    for (int e = q; e < E; e += LPT) row[e] = row[e] / z;
-  }
-
-  // top-k: each round, every lane offers its best remaining expert (ties: lowest id)
-  constexpr int TW = (EP + 32 * LPT - 1) / (32 * LPT);
-  uint32_t taken[TW];  // word c, bit b: expert q + LPT * (32 c + b)
-#pragma unroll
-  for (int c = 0; c < TW; ++c) taken[c] = 0;
   int* sel = sel_s[tid / LPT];
   float* val = val_s[tid / LPT];
-#pragma unroll 1
-  for (int j = 0; j < topk; ++j) {
-    float best = 0.0f;
-    int best_e = -1;
+  constexpr int EL = EP / LPT;  // experts a lane
+  if constexpr (EL <= 16) {
+    // A lane keeps its experts' values in registers: the rounds of the top-k then compare
+    // registers (a scan through LDS with a test and a read per expert and round was most of
+    // the kernel from 64 experts on).
+    // the reference's logits are a matmul result in the dtype of x (router.py:22); the
+    // Ernie router keeps them in fp32 (:44)
+    float p[EL], key[EL];
+    float mx = -INFINITY;
 #pragma unroll
-    for (int c = 0; c < TW; ++c) {
-      const uint32_t tk = taken[c];
+    for (int i = 0; i < EL; ++i) {
+      const int e = q + LPT * i;
+      float v = -INFINITY;
+      if (e < E) {
+        v = row[e];
+        if (!ernie && sizeof(TX) == 2) v = to_f32(from_f32<TX>(v));
+        if (g.logits_out != nullptr && t < g.T) g.logits_out[t * E + e] = v;
+      }
+      p[i] = v;
+      mx = fmaxf(mx, v);
+    }
+    mx = group_max(mx);
+    if (softmax_first) {
+      float z = 0.0f;
+#pragma unroll
+      for (int i = 0; i < EL; ++i) {
+        p[i] = q + LPT * i < E ? expf(p[i] - mx) : 0.0f;
+        z += p[i];
+      }
+      z = group_sum(z);
+#pragma unroll
+      for (int i = 0; i < EL; ++i) p[i] = p[i] / z;
+    }
+    // selection keys; an expert that is taken, or past E, can no longer win
+#pragma unroll
+    for (int i = 0; i < EL; ++i) {
+      const int e = q + LPT * i;
+      key[i] = e < E ? (ernie ? p[i] + g.bias[e] : p[i]) : -INFINITY;
+    }
+    // top-k: each round, every lane offers its best remaining expert (ties: lowest id)
 #pragma unroll 1
-      for (int b = 0, e = q + LPT * 32 * c; b < 32 && e < E; ++b, e += LPT) {
-        if (tk & (1u << b)) continue;
-        const float key = ernie ? row[e] + g.bias[e] : row[e];
-        if (best_e < 0 || key > best) {
-          best = key;
-          best_e = e;
-        }
+    for (int j = 0; j < topk; ++j) {
+      float best = -INFINITY, best_v = 0.0f;
+      int best_e = -1;
+#pragma unroll
+      for (int i = 0; i < EL; ++i) {
+        const bool take = key[i] > best || (best_e < 0 && q + LPT * i < E && key[i] != -INFINITY);
+        best_v = take ? p[i] : best_v;
+        best_e = take ? q + LPT * i : best_e;
+        best = take ? key[i] : best;
+      }
+#pragma unroll
+      for (int o = 1; o < LPT; o <<= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const float ov = __shfl_xor(best_v, o, 64);
+        const int oe = __shfl_xor(best_e, o, 64);
+        const bool take = oe >= 0 && (best_e < 0 || ob > best || (ob == best && oe < best_e));
+        best = take ? ob : best;
+        best_v = take ? ov : best_v;
+        best_e = take ? oe : best_e;
+      }
+      best_e = best_e < 0 ? 0 : best_e;  // only if topk > E, which the entry point rejects
+#pragma unroll
+      for (int i = 0; i < EL; ++i) key[i] = best_e == q + LPT * i ? -INFINITY : key[i];
+      if (q == 0) {
+        sel[j] = best_e;
+        val[j] = best_v;
       }
     }
-#pragma unroll
-    for (int o = 1; o < LPT; o <<= 1) {
-      const float ob = __shfl_xor(best, o, 64);
-      const int oe = __shfl_xor(best_e, o, 64);
-      const bool take = oe >= 0 && (best_e < 0 || ob > best || (ob == best && oe < best_e));
-      best = take ? ob : best;
-      best_e = take ? oe : best_e;
+  } else {
+    // the reference's logits are a matmul result in the dtype of x (router.py:22); the
+    // Ernie router keeps them in fp32 (:44)
+    float mx = -INFINITY;
+    for (int e = q; e < E; e += LPT) {
+      float v = row[e];
+      if (!ernie && sizeof(TX) == 2) v = to_f32(from_f32<TX>(v));
+      row[e] = v;
+      if (g.logits_out != nullptr && t < g.T) g.logits_out[t * E + e] = v;
+      mx = fmaxf(mx, v);
     }
-    best_e = best_e < 0 ? 0 : best_e;  // only if topk > E, which the entry point rejects
-    if (best_e % LPT == q) {
-      const int i = best_e / LPT;
-#pragma unroll
-      for (int c = 0; c < TW; ++c)
-        if ((i >> 5) == c) taken[c] |= 1u << (i & 31);
+    mx = group_max(mx);
+    if (softmax_first) {
+      float z = 0.0f;
+      for (int e = q; e < E; e += LPT) {
+        const float p = expf(row[e] - mx);
+        row[e] = p;
+        z += p;
+      }
+      z = group_sum(z);
+      for (int e = q; e < E; e += LPT) row[e] = row[e] / z;
     }
-    if (q == 0) {
-      sel[j] = best_e;
-      val[j] = row[best_e];
+
+    // top-k: each round, every lane offers its best remaining expert (ties: lowest id)
+    constexpr int TW = (EP + 32 * LPT - 1) / (32 * LPT);
+    uint32_t taken[TW];  // word c, bit b: expert q + LPT * (32 c + b)
+#pragma unroll
+    for (int c = 0; c < TW; ++c) taken[c] = 0;
+#pragma unroll 1
+    for (int j = 0; j < topk; ++j) {
+      float best = 0.0f;
+      int best_e = -1;
+#pragma unroll
+      for (int c = 0; c < TW; ++c) {
+        const uint32_t tk = taken[c];
+#pragma unroll 1
+        for (int b = 0, e = q + LPT * 32 * c; b < 32 && e < E; ++b, e += LPT) {
+          if (tk & (1u << b)) continue;
+          const float key = ernie ? row[e] + g.bias[e] : row[e];
+          if (best_e < 0 || key > best) {
+            best = key;
+            best_e = e;
+          }
+        }
+      }
+#pragma unroll
+      for (int o = 1; o < LPT; o <<= 1) {
+        const float ob = __shfl_xor(best, o, 64);
+        const int oe = __shfl_xor(best_e, o, 64);
+        const bool take = oe >= 0 && (best_e < 0 || ob > best || (ob == best && oe < best_e));
+        best = take ? ob : best;
+        best_e = take ? oe : best_e;
+      }
+      best_e = best_e < 0 ? 0 : best_e;  // only if topk > E, which the entry point rejects
+      if (best_e % LPT == q) {
+        const int i = best_e / LPT;
+#pragma unroll
+        for (int c = 0; c < TW; ++c)
+          if ((i >> 5) == c) taken[c] |= 1u << (i & 31);
+      }
+      if (q == 0) {
+        sel[j] = best_e;
+        val[j] = row[best_e];
+      }
     }
   }
   // (the lanes of a token sit in one wavefront: LDS writes above are visible below)
