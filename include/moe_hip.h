@@ -104,7 +104,12 @@ MOE_API int moe_route_preprocess(const void* expert_ids, int idx_bytes, int64_t 
  * moe_route_workspace_bytes(R, E) above that (ceil(R / 512) * E > 2^20) return
  * MOE_ERR_WORKSPACE.  All calls on one device share that buffer: calls that may overlap in
  * time (different streams) race; calls on one stream are ordered and safe.  Nothing in the
- * buffer has to be cleared between calls.
+ * buffer has to be cleared between calls.  Under graph capture the captured launches keep
+ * using that one buffer: replays of a graph that holds this call must not overlap each other
+ * or an eager call on the same device (replays launched into one stream are ordered and
+ * safe).  The first call on a device looks up the buffer's address and is refused with
+ * MOE_ERR_HIP while its stream is being captured: make one call (R = 0 will do) before the
+ * capture begins.
  */
 MOE_API size_t moe_route_noalloc_max_bytes(void);
 MOE_API int moe_route_preprocess_noalloc(const void* expert_ids, int idx_bytes, int64_t R, int E,

@@ -1,12 +1,6 @@
 """Builds libmoe_hip.so (the HIP kernels + C ABI) for gfx950 with hipcc.
 
     python moe-explore_amd/build.py [--jobs N] [--force]
-    python moe-explore_amd/build.py --ablate N --out /some/dir/libmoe_hip_ablate.so
-
-The second form builds a diagnostic copy of the library whose GEMM kernels leave parts of
-their K loop out (-DMOE_ABLATE=N, see csrc/gemm_mfma_dma.hip and csrc/gemm_kgrouped.hip): wrong
-results, used only to time what a K step spends on what (MOE_HIP_LIB=<that file> bench.py
---only ablation).  It never touches moe_explore/libmoe_hip.so.
 
 Each csrc/*.hip is compiled to an object under build/ and the objects are linked
 into moe_explore/libmoe_hip.so.  Nothing is compiled at import time: the Python
@@ -88,47 +82,9 @@ def build(jobs=None, force=False, verbose=True, extra=()):
     return LIB
 
 
-def build_ablation(mask, out):
-    """Diagnostic library: the two GEMM sources compiled with -DMOE_ABLATE=mask, linked with the
-    product build's other objects into `out` (which must not be the product library)."""
-    out = os.path.abspath(out)
-    assert out != os.path.abspath(LIB), "an ablation build never replaces the product library"
-    build(verbose=False)
-    os.makedirs(os.path.dirname(out), exist_ok=True)
-    tmp = out + ".objs"
-    os.makedirs(tmp, exist_ok=True)
-    swapped = ("gemm_mfma_dma", "gemm_kgrouped")
-    objs = [os.path.join(BUILD, f[:-4] + ".o") for f in sorted(os.listdir(CSRC))
-            if f.endswith(".hip") and f[:-4] not in swapped]
-    for name in swapped:
-        obj = os.path.join(tmp, name + ".o")
-        _, rc, log = _compile(os.path.join(CSRC, name + ".hip"), obj, [f"-DMOE_ABLATE={int(mask)}"])
-        if rc != 0:
-            print(log, file=sys.stderr)
-            raise RuntimeError("hipcc failed")
-        objs.append(obj)
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out,
-           "-Wl,-rpath,/opt/rocm/lib", "-Wl,--no-undefined"]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    shutil.rmtree(tmp, ignore_errors=True)
-    if r.returncode != 0:
-        print(r.stdout + r.stderr, file=sys.stderr)
-        raise RuntimeError("link failed")
-    print(f"[build] ablation {mask}: {out}")
-    return out
-
-
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=None)
     ap.add_argument("--force", action="store_true")
-    ap.add_argument("--ablate", type=int, default=None, metavar="MASK",
-                    help="build a diagnostic library with -DMOE_ABLATE=MASK instead (needs --out)")
-    ap.add_argument("--out", default=None, help="path of the ablation library")
     a = ap.parse_args()
-    if a.ablate is not None:
-        if not a.out:
-            ap.error("--ablate needs --out")
-        build_ablation(a.ablate, a.out)
-    else:
-        build(jobs=a.jobs, force=a.force)
+    build(jobs=a.jobs, force=a.force)

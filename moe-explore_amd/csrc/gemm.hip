@@ -2,20 +2,7 @@
 // MFMA kernels and the scalar-FMA kernel.
 #include "gemm.h"
 
-#include <stdlib.h>
-
 using namespace moe;
-
-namespace {
-// MOE_HIP_FORCE_SCALAR=1 routes every GEMM to the scalar-FMA kernels (debugging).
-bool force_scalar() {
-  static const bool v = [] {
-    const char* s = getenv("MOE_HIP_FORCE_SCALAR");
-    return s != nullptr && s[0] == '1';
-  }();
-  return v;
-}
-}  // namespace
 
 extern "C" int moe_m_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, const void* w,
                                   int64_t ldw_e, int64_t ldw_k, int64_t ldw_n, void* c,
@@ -40,12 +27,13 @@ extern "C" int moe_m_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
   const bool glu = act_is_glu(epilogue);
   MOE_REQUIRE(!glu || N % 2 == 0, "a GLU epilogue needs an even N, got %lld", (long long)N);
   MOE_REQUIRE(group_indices != nullptr, "group_indices is null");
-  if (gather || scatter || scatter_add) {
-    MOE_REQUIRE(indices != nullptr, "gather/scatter needs indices");
-    MOE_REQUIRE(idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8, got %d", idx_bytes);
-  }
   const int64_t P = gather ? c_rows : a_rows;
   MOE_REQUIRE(P <= 0x7fffffff, "too many rows");
+  if (gather || scatter || scatter_add) {
+    // (an empty batch has an empty index array, whose pointer may be null)
+    MOE_REQUIRE(indices != nullptr || P == 0, "gather/scatter needs indices");
+    MOE_REQUIRE(idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8, got %d", idx_bytes);
+  }
   if (P == 0 || N == 0) return MOE_OK;
   MOE_REQUIRE(a != nullptr && w != nullptr && c != nullptr, "null operand");
   MOE_REQUIRE(a_rows > 0 && c_rows > 0, "empty operand with non-empty groups");
@@ -63,7 +51,7 @@ extern "C" int moe_m_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
     // split K: only the direct-to-LDS MFMA kernel, and only where partial sums can be
     // added afterwards (no epilogue, plain or row-scatter store)
     MOE_REQUIRE(ksplit <= 8, "ksplit must be in [1,8], got %d", ksplit);
-    if (epilogue != MOE_ACT_NONE || save || scatter_add || force_scalar() ||
+    if (epilogue != MOE_ACT_NONE || save || scatter_add ||
         !m_grouped_mfma_supported(g) || K % (64 * ksplit) != 0)
       return fail(MOE_ERR_UNSUPPORTED, "split K needs the MFMA kernel, no epilogue and K %% (64*ksplit) == 0");
     MOE_REQUIRE(c_split_stride >= (c_rows - 1) * ldc + N, "c_split_stride smaller than one copy of c");
@@ -75,8 +63,8 @@ extern "C" int moe_m_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
   const bool copy_preact = save && epilogue == MOE_ACT_NONE && !scatter && !scatter_add;
   if (copy_preact) g.flags &= ~MOE_GEMM_SAVE_PREACT;
   int rc;
-  if (!force_scalar() && m_grouped_mfma_supported(g)) rc = launch_m_grouped_mfma(g, s);
-  else if (!force_scalar() && m_grouped_f32_mfma_supported(g)) rc = launch_m_grouped_f32_mfma(g, s);
+  if (m_grouped_mfma_supported(g)) rc = launch_m_grouped_mfma(g, s);
+  else if (m_grouped_f32_mfma_supported(g)) rc = launch_m_grouped_f32_mfma(g, s);
   else rc = launch_m_grouped_generic(g, s);
   if (rc != MOE_OK || !copy_preact) return rc;
   const size_t esz = dtype_bytes(dtype);
@@ -105,7 +93,7 @@ extern "C" int moe_m_grouped_gemm_glu_bwd(const void* a, int64_t a_rows, int64_t
   MOE_REQUIRE((flags & ~MOE_GEMM_GATHER_A) == 0, "only MOE_GEMM_GATHER_A is allowed, got 0x%x", flags);
   MOE_REQUIRE(group_indices != nullptr, "group_indices is null");
   MOE_REQUIRE(indices == nullptr || idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8");
-  MOE_REQUIRE(!(flags & MOE_GEMM_GATHER_A) || indices != nullptr, "GATHER_A needs indices");
+  MOE_REQUIRE(!(flags & MOE_GEMM_GATHER_A) || indices != nullptr || P == 0, "GATHER_A needs indices");
   MOE_REQUIRE(P <= 0x7fffffff, "too many rows");
   if (P == 0 || N == 0) return MOE_OK;
   MOE_REQUIRE(a && w && h && dh && y_scaled, "null operand");
@@ -118,7 +106,7 @@ extern "C" int moe_m_grouped_gemm_glu_bwd(const void* a, int64_t a_rows, int64_t
   g.h = h;
   g.ldh = ldh;
   g.dscale = dscale;
-  if (force_scalar() || !m_grouped_mfma_supported(g) || !m_grouped_mfma_dma_supported(g) ||
+  if (!m_grouped_mfma_supported(g) || !m_grouped_mfma_dma_supported(g) ||
       !(g.ldw_k == 1 && g.ldw_n % 8 == 0))
     return fail(MOE_ERR_UNSUPPORTED, "fused GLU backward: needs the direct-to-LDS MFMA kernel with "
                                      "K-contiguous weights (K %% 64 == 0, aligned rows)");
@@ -142,7 +130,8 @@ extern "C" int moe_k_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
               "at most one operand is K-major, and then nothing is gathered");
   MOE_REQUIRE(group_indices != nullptr, "group_indices is null");
   if (ga || gb) {
-    MOE_REQUIRE(indices != nullptr, "gather needs indices");
+    // (an empty batch has an empty index array, whose pointer may be null)
+    MOE_REQUIRE(indices != nullptr || (ga ? b_rows : a_rows) == 0, "gather needs indices");
     MOE_REQUIRE(idx_bytes == 4 || idx_bytes == 8, "idx_bytes must be 4 or 8, got %d", idx_bytes);
   }
   if (Ka == 0 || Nb == 0) return MOE_OK;
@@ -164,8 +153,8 @@ extern "C" int moe_k_grouped_gemm(const void* a, int64_t a_rows, int64_t lda, co
   KGemmArgs g{a, a_rows, lda, b, b_rows, ldb, out, group_indices, indices, idx_bytes,
               E, Ka,     Nb,  topk, flags, dtype, P, FastDiv(static_cast<uint32_t>(topk))};
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (!force_scalar() && k_grouped_mfma_supported(g)) return launch_k_grouped_mfma(g, s);
-  if (!force_scalar() && k_grouped_f32_mfma_supported(g)) return launch_k_grouped_f32_mfma(g, s);
+  if (k_grouped_mfma_supported(g)) return launch_k_grouped_mfma(g, s);
+  if (k_grouped_f32_mfma_supported(g)) return launch_k_grouped_f32_mfma(g, s);
   if (ka || kb)
     return fail(MOE_ERR_UNSUPPORTED, "K-major operands need the MFMA kernel (16-bit dtype, widths and "
                                      "strides multiples of 8, 16-byte aligned pointers)");

@@ -26,12 +26,6 @@
 // read through transpose loads the LDS, not the matrix cores, sets the pace of a K step.
 #include "gemm_mfma.h"
 
-// Ablation builds (`build.py --ablate N`; never the product library, results are wrong): bit 1
-// skips the a-fragment LDS reads of the K loop, bit 2 the b-fragment reads.
-#ifndef MOE_ABLATE
-#define MOE_ABLATE 0
-#endif
-
 #include <mutex>
 #include <set>
 #include <utility>
@@ -550,18 +544,18 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
       if (more) issue_short(sstage ^ 1);
       __builtin_amdgcn_s_setprio(2);
       __builtin_amdgcn_sched_barrier(0);
-      if (!(MOE_ABLATE & 2)) read_unit_b(sstage, lstage, 0, 1, bfP);
-      if (!(MOE_ABLATE & 1)) read_unit_a(sstage, lstage, 1, afB);
+      read_unit_b(sstage, lstage, 0, 1, bfP);
+      read_unit_a(sstage, lstage, 1, afB);
       multiply_unit(0, afA, bfP);
       interleave_unit();
-      if (!(MOE_ABLATE & 2)) read_unit_b(sstage, lstage, 1, 0, bfQ);
-      if (!(MOE_ABLATE & 1)) read_unit_a(sstage, lstage, 2, afA);
+      read_unit_b(sstage, lstage, 1, 0, bfQ);
+      read_unit_a(sstage, lstage, 2, afA);
       multiply_unit(1, afB, bfP);
       interleave_unit();
       if (ahead) issue_long(lahead);
       __builtin_amdgcn_sched_barrier(0);
-      if (!(MOE_ABLATE & 2)) read_unit_b(sstage, lstage, 1, 1, bfQ);
-      if (!(MOE_ABLATE & 1)) read_unit_a(sstage, lstage, 3, afB);
+      read_unit_b(sstage, lstage, 1, 1, bfQ);
+      read_unit_a(sstage, lstage, 3, afB);
       multiply_unit(0, afA, bfQ);
       interleave_unit();
       __builtin_amdgcn_s_setprio(0);
@@ -570,8 +564,8 @@ __global__ __launch_bounds__(kThreads) void k_grouped_persistent_kernel(KGemmArg
         // copy instructions of this wavefront, may still fly
         if (ahead) wait_copies_keep_youngest_and_barrier<4>();
         else wait_copies_and_barrier();
-        if (!(MOE_ABLATE & 1)) read_unit_a(sstage ^ 1, lnext, 0, afA);
-        if (!(MOE_ABLATE & 2)) read_unit_b(sstage ^ 1, lnext, 0, 0, bfP);
+        read_unit_a(sstage ^ 1, lnext, 0, afA);
+        read_unit_b(sstage ^ 1, lnext, 0, 0, bfP);
       }
       multiply_unit(1, afB, bfQ);
       interleave_unit();

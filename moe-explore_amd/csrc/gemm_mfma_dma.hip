@@ -29,18 +29,6 @@
 // layouts are applied to the global source address of each lane instead.
 #include "gemm_mfma.h"
 
-#include <stdlib.h>
-
-// Ablation builds (`build.py --ablate N`; never the product library): parts of the K loop
-// are left out, the results are wrong and only the run time is of interest.  It answers what a
-// K step spends on what: bit 1 skips half of the token-fragment LDS reads, 8 all of them, 4
-// the weight-fragment reads, 2 the global -> LDS copies of the loop, 16 / 32 make the token /
-// weight copies cycle through eight K steps (an L2-resident window: same LDS traffic, no
-// fabric or HBM traffic).  0 compiles to the product kernel, instruction for instruction.
-#ifndef MOE_ABLATE
-#define MOE_ABLATE 0
-#endif
-
 #include <mutex>
 #include <unordered_map>
 
@@ -128,7 +116,7 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
   const int KT = static_cast<int>(g.K / BK) / s.ksplit;  // K steps of this part
   const int kt0 = kpart * KT;
   g.c = static_cast<char*>(g.c) + static_cast<int64_t>(kpart) * g.c_split_stride * sizeof(T);
-  if (threadIdx.x < 64) find_tile<BM>(g.group_indices, g.E, static_cast<int>(g.P), mt, sh_tile);
+  if (threadIdx.x < 64) find_tile<BM, true>(g.group_indices, g.E, static_cast<int>(g.P), mt, sh_tile);
   __syncthreads();
   const int expert = __builtin_amdgcn_readfirstlane(sh_tile[0]);
   if (expert < 0) return;
@@ -203,7 +191,7 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
 #pragma unroll
     for (int i = 0; i < A_INSTR; ++i)
       if (i >= first && i < last && 8 * (NWAVES * i + wave) < rows_here)
-        copy16_to_lds(g.a, a_src[i] + static_cast<uint32_t>((MOE_ABLATE & 16) ? ((kt0 + kt) & 7) : (kt0 + kt)) * (BK * 2),
+        copy16_to_lds(g.a, a_src[i] + static_cast<uint32_t>(kt0 + kt) * (BK * 2),
                       base + i * (NWAVES * 1024));
   };
   auto issue_weight_copies = [&](int wstage, int kt, int first, int last) __attribute__((always_inline)) {
@@ -211,7 +199,7 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
 #pragma unroll
     for (int i = 0; i < W_INSTR; ++i)
       if (i >= first && i < last)
-        copy16_to_lds(wbase, w_src[i] + static_cast<uint32_t>((MOE_ABLATE & 32) ? ((kt0 + kt) & 7) : (kt0 + kt)) * w_step,
+        copy16_to_lds(wbase, w_src[i] + static_cast<uint32_t>(kt0 + kt) * w_step,
                       base + i * (NWAVES * 1024));
   };
 
@@ -357,30 +345,30 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
       const int wahead = wnext == 2 ? 0 : wnext + 1;
       const bool more = gs + 1 < S, ahead = gs + 2 < S;
       const bool tile_ends = kt + 1 == KT;
-      if (more && !(MOE_ABLATE & 2)) issue_token_copies(stage ^ 1, kt_a, 0, AH);
+      if (more) issue_token_copies(stage ^ 1, kt_a, 0, AH);
       __builtin_amdgcn_s_setprio(2);
       __builtin_amdgcn_sched_barrier(0);
-      if (!(MOE_ABLATE & 4)) read_unit_w(wcur, 0, 1, wfP, blocks);
-      if (!(MOE_ABLATE & 9)) read_unit_t(stage, 1, tfB, blocks);
+      read_unit_w(wcur, 0, 1, wfP, blocks);
+      read_unit_t(stage, 1, tfB, blocks);
       multiply_unit(0, tfA, wfP, blocks);
       interleave_unit();
       if (more) {
-        if (!(MOE_ABLATE & 2)) issue_token_copies(stage ^ 1, kt_a, AH, A_INSTR);
+        issue_token_copies(stage ^ 1, kt_a, AH, A_INSTR);
         advance_a();
       }
       __builtin_amdgcn_sched_barrier(0);
-      if (!(MOE_ABLATE & 4)) read_unit_w(wcur, 1, 0, wfQ, blocks);
-      if (!(MOE_ABLATE & 8)) read_unit_t(stage, 2, tfA, blocks);
+      read_unit_w(wcur, 1, 0, wfQ, blocks);
+      read_unit_t(stage, 2, tfA, blocks);
       multiply_unit(1, tfB, wfP, blocks);
       interleave_unit();
-      if (ahead && !(MOE_ABLATE & 2)) issue_weight_copies(wahead, kt_w, 0, WH);
+      if (ahead) issue_weight_copies(wahead, kt_w, 0, WH);
       __builtin_amdgcn_sched_barrier(0);
-      if (!(MOE_ABLATE & 4)) read_unit_w(wcur, 1, 1, wfQ, blocks);
-      if (!(MOE_ABLATE & 9)) read_unit_t(stage, 3, tfB, blocks);
+      read_unit_w(wcur, 1, 1, wfQ, blocks);
+      read_unit_t(stage, 3, tfB, blocks);
       multiply_unit(0, tfA, wfQ, blocks);
       interleave_unit();
       if (ahead) {
-        if (!(MOE_ABLATE & 2)) issue_weight_copies(wahead, kt_w, WH, W_INSTR);
+        issue_weight_copies(wahead, kt_w, WH, W_INSTR);
         advance_w();
       }
       __builtin_amdgcn_s_setprio(0);
@@ -392,8 +380,8 @@ __device__ __forceinline__ void m_grouped_dma_tile(MGemmArgs g, const Sched s, c
         // (the first fragments of a next tile are read after the store of this one:
         // held across the store they would crowd the register file)
         if (!tile_ends) {
-          if (!(MOE_ABLATE & 8)) read_unit_t(stage ^ 1, 0, tfA, blocks);
-          if (!(MOE_ABLATE & 4)) read_unit_w(wnext, 0, 0, wfP, blocks);
+          read_unit_t(stage ^ 1, 0, tfA, blocks);
+          read_unit_w(wnext, 0, 0, wfP, blocks);
         }
       }
       multiply_unit(1, tfB, wfQ, blocks);
@@ -567,9 +555,8 @@ template <typename T, int BM, int WVM, int WVN, int WL>
 int launch_act(const MGemmArgs& g, hipStream_t stream) {
   // two column tiles a workgroup where that still leaves several rounds of workgroups
   const int64_t tiles = ((g.P + BM - 1) / BM + g.E / 2) * ((g.N + BN - 1) / BN) * (g.ksplit < 1 ? 1 : g.ksplit);
-  static const int forced_tpw = [] { const char* e = getenv("MOE_HIP_TPW"); return e ? atoi(e) : 0; }();
   // (the fused GLU backward stores through the whole LDS: one column tile a workgroup)
-  const int tpw = (g.flags & MOE_GEMM_GLU_BWD) ? 1 : (forced_tpw > 0 ? forced_tpw : (tiles >= 2048 ? 2 : 1));
+  const int tpw = (g.flags & MOE_GEMM_GLU_BWD) ? 1 : (tiles >= 2048 ? 2 : 1);
   Sched s = make_sched(g, BM, tpw);
   if (s.wgs > 0x7fffffff) return fail(MOE_ERR_UNSUPPORTED, "grid too large");
   // 2 token + 3 weight stages; BM = 128 adds room for the store staging of half the wavefronts

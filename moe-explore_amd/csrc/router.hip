@@ -279,11 +279,15 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
 #pragma unroll
       for (int i = 0; i < EL; ++i) p[i] = p[i] / z;
     }
-    // selection keys; an expert that is taken, or past E, can no longer win
+    // selection keys, and a bit per expert of this lane that can still win: set for the experts
+    // below E, cleared when one is taken (a key itself may be -inf: a masked logit with the
+    // top-k first; it is then chosen after every finite one, lowest id first, as torch.topk does)
+    uint32_t open = 0;
 #pragma unroll
     for (int i = 0; i < EL; ++i) {
       const int e = q + LPT * i;
       key[i] = e < E ? (ernie ? p[i] + g.bias[e] : p[i]) : -INFINITY;
+      open |= e < E ? (1u << i) : 0u;
     }
     // top-k: each round, every lane offers its best remaining expert (ties: lowest id)
 #pragma unroll 1
@@ -292,7 +296,7 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
       int best_e = -1;
 #pragma unroll
       for (int i = 0; i < EL; ++i) {
-        const bool take = key[i] > best || (best_e < 0 && q + LPT * i < E && key[i] != -INFINITY);
+        const bool take = ((open >> i) & 1u) && (best_e < 0 || key[i] > best);
         best_v = take ? p[i] : best_v;
         best_e = take ? q + LPT * i : best_e;
         best = take ? key[i] : best;
@@ -309,7 +313,7 @@ __global__ __launch_bounds__(512) void router_fwd_kernel(RouterArgs g) {
       }
       best_e = best_e < 0 ? 0 : best_e;  // only if topk > E, which the entry point rejects
 #pragma unroll
-      for (int i = 0; i < EL; ++i) key[i] = best_e == q + LPT * i ? -INFINITY : key[i];
+      for (int i = 0; i < EL; ++i) open &= best_e == q + LPT * i ? ~(1u << i) : ~0u;
       if (q == 0) {
         sel[j] = best_e;
         val[j] = best_v;

@@ -215,7 +215,10 @@ int check_route_args(const void* expert_ids, int idx_bytes, int64_t R, int E,
 constexpr size_t kScratchWords = size_t(1) << 20;  // 4 MiB
 static __device__ __align__(256) int32_t scratch[kScratchWords];
 
-int32_t* scratch_of_current_device() {
+// `stream`: the stream of the call that asks.  The first call on a device looks the address up
+// (which may load the code object); that is not done while `stream` is being captured into a
+// graph: such a call is refused, and the caller makes one call outside the capture first.
+int32_t* scratch_of_current_device(hipStream_t stream) {
   constexpr int kMaxDevices = 64;
   static int32_t* of_device[kMaxDevices];
   static std::mutex lock;
@@ -227,6 +230,18 @@ int32_t* scratch_of_current_device() {
   }
   std::lock_guard<std::mutex> hold(lock);
   if (of_device[dev] == nullptr) {
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    err = hipStreamIsCapturing(stream, &capture);
+    if (err != hipSuccess) {
+      fail(MOE_ERR_HIP, "hipStreamIsCapturing: %s", hipGetErrorString(err));
+      return nullptr;
+    }
+    if (capture != hipStreamCaptureStatusNone) {
+      fail(MOE_ERR_HIP, "the first moe_route_preprocess_noalloc call on a device looks up its "
+                        "resident buffer and cannot run under stream capture: make one call "
+                        "(any size, R = 0 will do) before the capture begins");
+      return nullptr;
+    }
     void* p = nullptr;
     err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (err != hipSuccess || p == nullptr) {
@@ -270,7 +285,7 @@ extern "C" int moe_route_preprocess_noalloc(const void* expert_ids, int idx_byte
                 "routing of %lld slots over %d experts needs %zu bytes of scratch; the resident "
                 "buffer of moe_route_preprocess_noalloc has %zu (use moe_route_preprocess with a "
                 "workspace)", (long long)R, E, need, kScratchWords * sizeof(int32_t));
-  int32_t* const counts = scratch_of_current_device();
+  int32_t* const counts = scratch_of_current_device(static_cast<hipStream_t>(stream_));
   if (counts == nullptr) return MOE_ERR_HIP;
   return route_preprocess_launch(expert_ids, idx_bytes, R, E, indices_out, group_indices_out,
                                  inclusive_out, counts, static_cast<hipStream_t>(stream_));

@@ -10,8 +10,6 @@ gradient; the reference itself is forward-only.
 ``topk_moe_torch`` is the plain-PyTorch per-expert loop that the reference ships
 as its comparison implementation (``:67-102``); it is not used by the HIP path.
 """
-import weakref
-
 import torch
 
 from moe_explore.params import MOEParams, MLPParams, GLUParams, GLUInterleavedParams
@@ -51,36 +49,13 @@ def to_interleaved(ep):
     return ep
 
 
-# interleaved copies of GLUParams weights, one per (gate, up) pair, rebuilt only when one of
-# the two tensors has been written since (their version counters)
-_interleaved_cache = {}
-_INTERLEAVED_CACHE_MAX = 256
-
-
-def _cached_interleave(gate, up):
-    key = (id(gate), id(up))
-    hit = _interleaved_cache.get(key)
-    if hit is not None:
-        g_ref, u_ref, g_ver, u_ver, ptrs, w = hit
-        if g_ref() is gate and u_ref() is up and g_ver == gate._version and \
-                u_ver == up._version and ptrs == (gate.data_ptr(), up.data_ptr()):
-            return w
-    w = interleave_glu_weights(gate.detach(), up.detach())
-    if len(_interleaved_cache) >= _INTERLEAVED_CACHE_MAX:
-        _interleaved_cache.clear()
-    drop = lambda _, key=key: _interleaved_cache.pop(key, None)
-    _interleaved_cache[key] = (weakref.ref(gate, drop), weakref.ref(up, drop), gate._version,
-                               up._version, (gate.data_ptr(), up.data_ptr()), w)
-    return w
-
-
 class _InterleaveFunction(torch.autograd.Function):
-    """Differentiable view of the cached interleaved copy: the gradient of weight1 goes
-    back to gate and up as its even and odd columns."""
+    """Differentiable interleave: the gradient of weight1 goes back to gate and up as its
+    even and odd columns."""
 
     @staticmethod
     def forward(ctx, gate, up):
-        return _cached_interleave(gate, up).detach()
+        return interleave_glu_weights(gate, up)
 
     @staticmethod
     def backward(ctx, dw):
@@ -89,8 +64,10 @@ class _InterleaveFunction(torch.autograd.Function):
 
 def expert_weights(ep):
     """(weight1, weight2, activation) of any of the reference's FFN parameter records.
-    Separate gate / up weights are interleaved once and the copy is reused until either
-    tensor is written again."""
+    Separate gate / up weights are interleaved on every call (one pass over the two tensors):
+    no copy is kept between calls, because nothing a tensor exposes tells whether its storage
+    has been written since (updates through ``.data``, graph replays and raw kernels leave the
+    version counter alone).  ``to_interleaved`` converts once, at load time."""
     if isinstance(ep, MLPParams):
         return ep.weight1, ep.weight2, ep.activation
     if isinstance(ep, GLUInterleavedParams):
@@ -100,7 +77,7 @@ def expert_weights(ep):
         if torch.is_grad_enabled() and (gate.requires_grad or up.requires_grad):
             w1 = _InterleaveFunction.apply(gate, up)
         else:
-            w1 = _cached_interleave(gate, up)
+            w1 = interleave_glu_weights(gate.detach(), up.detach())
         return w1, ep.down_weight, glu_form(ep.activation)
     raise ValueError(f"Unsupported expert parameter type: {type(ep)}")
 
@@ -118,6 +95,38 @@ def _ksplit_for(rows, num_experts, n, k):
 
 # intermediate width below which the dW2 kernel gathers its token rows itself (see backward)
 _FUSED_GATHER_BELOW_FF = 1280
+
+
+def _dw2(a_scaled, dout, gi, idx, topk):
+    """dW2 = (s*A)^T dOut over every expert's positions.  The token rows are gathered first,
+    feature-major (one 25 us pass over R x d): the K-grouped kernel then reads that operand from
+    LDS with plain 16-byte loads instead of transpose loads.  The kernel can also gather by
+    itself, but then has to wait for the row ids of every K step, and with them for the copies
+    it keeps in flight: 10-15 % slower.  That is still the cheaper way for narrow experts: the
+    pass over R x d costs ~330 / ff of the GEMM it serves (ff = 1024: a third), so below
+    ff = 1280 the kernel gathers dout itself (OLMoE shape, T = 8192: 0.362 -> 0.316 ms; Qwen3
+    shape, T = 32000: 1.09 -> 0.91 ms; ff = 1408 the same either way)."""
+    if a_scaled.size(1) < _FUSED_GATHER_BELOW_FF:
+        return k_grouped_gemm(a_scaled, dout, gi, idx, topk, gather_b=True)
+    dw2 = None
+    dt = row_gather_kmajor(dout, idx, topk, gi)
+    if dt is not None:
+        dw2 = k_grouped_gemm(a_scaled, dt, gi, b_kmajor=True)
+    if dw2 is None:  # a shape the feature-major path does not take
+        dw2 = k_grouped_gemm(a_scaled, row_gather(dout, idx, topk), gi)
+    return dw2
+
+
+def _dw1(x, dh, gi, idx, topk):
+    """dW1 = Xg^T dH; the gathered token rows feature-major where the kernel takes them (-10 %
+    at the Mixtral shape; its GEMM is twice as long as dW2's, so it always gathers first)."""
+    dw1 = None
+    xt = row_gather_kmajor(x, idx, topk, gi)
+    if xt is not None:
+        dw1 = k_grouped_gemm(xt, dh, gi, a_kmajor=True)
+    if dw1 is None:
+        dw1 = k_grouped_gemm(row_gather(x, idx, topk), dh, gi)
+    return dw1
 
 
 class _ExpertsFunction(torch.autograd.Function):
@@ -141,7 +150,7 @@ class _ExpertsFunction(torch.autograd.Function):
         ks = _ksplit_for(T * topk, w2.size(0), w2.size(2), w2.size(1))
         with scope("down_grouped_gemm"):
             y = m_grouped_gemm(a, p2, ksplit=ks)
-        ks = y.size(0) // (T * topk)
+        ks = y.size(0) // (T * topk) if T else 1
         with scope("scale_and_reduce"):
             out = scale_and_reduce(y, scores, T, topk, y.size(1), nsplit=ks)
         if need_grad:
@@ -171,34 +180,20 @@ class _ExpertsFunction(torch.autograd.Function):
             dh, a_scaled, dscale = act_bwd(h, g, act, row_scale=scores, permute_indices=idx,
                                            want_y_scaled=True, want_dscale=need_dscore)
         dw1 = dw2 = dx = dscores = None
-        # Weight gradients: the token rows are gathered first, feature-major (one 25 us pass
-        # over R x d each): the K-grouped kernel then reads that operand from LDS with plain
-        # 16-byte loads instead of transpose loads (-10 % on dW1 at the Mixtral shape).  The
-        # kernel can also gather by itself, but then has to wait for the row ids of every K
-        # step, and with them for the copies it keeps in flight: 10-15 % slower.  That is still
-        # the cheaper way for dW2 of narrow experts: the pass over R x d costs ~330 / ff of the
-        # GEMM it serves (ff = 1024: a third), so below ff = 1280 the kernel gathers dout itself
-        # (OLMoE shape, T = 8192: 0.362 -> 0.316 ms; Qwen3 shape, T = 32000: 1.09 -> 0.91 ms;
-        # ff = 1408 the same either way; dW1, whose GEMM is twice as long, gathers first).
+        # dW2, dW1 and dX share no output, but they run one after the other on the calling stream:
+        # forked onto side streams of equal priority the hardware deals the compute units out
+        # among the three resident-workgroup launches from the start (not only in the last
+        # round of each), the launches lose the L2 locality of their tile order, and the step
+        # is 8 % slower (Mixtral shape: 8.76 -> 9.5 ms).
         if ctx.needs_input_grad[2]:
-            dt = None if a_scaled.size(1) < _FUSED_GATHER_BELOW_FF else row_gather_kmajor(dout, idx, topk, gi)
-            if dt is not None:
-                dw2 = k_grouped_gemm(a_scaled, dt, gi, b_kmajor=True)
-            elif a_scaled.size(1) < _FUSED_GATHER_BELOW_FF:
-                dw2 = k_grouped_gemm(a_scaled, dout, gi, idx, topk, gather_b=True)
-            else:
-                dw2 = k_grouped_gemm(a_scaled, row_gather(dout, idx, topk), gi)
+            dw2 = _dw2(a_scaled, dout, gi, idx, topk)
         if ctx.needs_input_grad[1]:
-            xt = row_gather_kmajor(x, idx, topk, gi)
-            if xt is not None:
-                dw1 = k_grouped_gemm(xt, dh, gi, a_kmajor=True)
-            else:
-                dw1 = k_grouped_gemm(row_gather(x, idx, topk), dh, gi)
+            dw1 = _dw1(x, dh, gi, idx, topk)
         if ctx.needs_input_grad[0]:
             px = MGroupedGEMMParams(w1, gi, idx, False, True, T, topk, scales=None)
             ks = _ksplit_for(T * topk, w1.size(0), w1.size(1), w1.size(2))
             dxg = m_grouped_gemm(dh, px, transpose_weight=True, ksplit=ks)
-            ks = dxg.size(0) // (T * topk)
+            ks = dxg.size(0) // (T * topk) if T else 1
             dx = scale_and_reduce(dxg, None, T, topk, dxg.size(1), nsplit=ks)
         if need_dscore:
             dscores = dscale.view(scores.shape).to(scores.dtype)

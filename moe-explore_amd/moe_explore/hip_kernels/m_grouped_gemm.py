@@ -190,8 +190,10 @@ def k_grouped_gemm(
     expert ``e``'s sorted positions.  ``gather_a`` / ``gather_b`` read that operand's
     row for position ``p`` at ``permute_indices[p] // topk``.  ``a_kmajor`` / ``b_kmajor``:
     that operand is the feature-major matrix ``row_gather_kmajor`` returns (the fast path
-    for the gathered token rows).  No reference counterpart (the reference is
-    forward-only)."""
+    for the gathered token rows); only the MFMA kernel reads that layout, and when it does not
+    take the shape (widths or strides not multiples of 8, unaligned pointers, no positions)
+    the call returns ``None`` and the caller gathers with ``row_gather`` instead.  No
+    reference counterpart (the reference is forward-only)."""
     assert a.dim() == 2 and b.dim() == 2 and a.dtype == b.dtype
     assert not (gather_a and gather_b) and not (a_kmajor and b_kmajor)
     assert not ((a_kmajor or b_kmajor) and (gather_a or gather_b))
@@ -220,6 +222,8 @@ def k_grouped_gemm(
         b.size(1) if b_kmajor else b.size(0), b.stride(0), out.data_ptr(),
         gi.data_ptr(), _C.ptr(perm), 0 if perm is None else _C.idx_bytes(perm), e, ka,
         nb, topk, flags, _C.dtype_code(a.dtype), _C.stream_of(a))
+    if st == -2 and (a_kmajor or b_kmajor):  # MOE_ERR_UNSUPPORTED
+        return None
     _C.check(st, "moe_k_grouped_gemm")
     return out
 

@@ -139,12 +139,13 @@ def config4_weights():
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("T,checked", [(128, 32), (1024, 48)])
+@pytest.mark.parametrize("T,checked", [(128, 32), (1024, 48), (8192, 32)])
 @pytest.mark.parametrize("act", ["swiglu", "geglu"])
 def test_fp8_layer_full_width_against_bf16_weights(config4_weights, T, checked, act):
-    """Config 4 at its real width, T = 128 and 1024 (the weight-streaming regime: split-K down
-    projection, tile-major weights): the fp8 layer against the fp32 oracle on the unquantised
-    weights for a subset of tokens (a token's output depends on its own row), <= 8e-2."""
+    """Config 4 at its real width: T = 128 and 1024 (the weight-streaming regime: split-K down
+    projection, tile-major weights) and T = 8192 (256-row tiles, bound by the matrix cores): the
+    fp8 layer against the fp32 oracle on the unquantised weights for a subset of tokens (a
+    token's output depends on its own row), <= 8e-2."""
     from moe_explore.fp8 import Fp8MLPParams, routed_experts_fp8
     q1, q2, (w1, w2) = config4_weights
     g = seeded(T + len(act))
@@ -159,7 +160,7 @@ def test_fp8_layer_full_width_against_bf16_weights(config4_weights, T, checked, 
     assert err <= 8e-2, f"fp8 layer, T={T}, {act}: rel-Frobenius {err:.3e} vs the bf16-weight oracle"
 
 
-@pytest.mark.parametrize("T", [128, 1024])
+@pytest.mark.parametrize("T", [128, 1024, 8192])
 def test_fp8_gate_up_gemm_full_width_against_dequantised_oracle(config4_weights, T):
     """The gate/up fp8 GEMM alone at full width (N = 28672, tile-major weights) against fp32
     products of the SAME codes and scales: rows of two experts, every column."""
@@ -176,13 +177,15 @@ def test_fp8_gate_up_gemm_full_width_against_dequantised_oracle(config4_weights,
     gi, ind = p.group_indices.cpu(), p.indices.cpu()
     xd = xq.cpu().float() * xs.cpu().unsqueeze(1)
     for e in (0, E - 1):
-        lo, hi = int(gi[e]), min(int(gi[e + 1]), int(gi[e]) + 24)
+        lo, hi = int(gi[e]), int(gi[e + 1])
         if hi <= lo:
             continue
+        # 24 positions spread over the expert's segment (every row block of it at T = 8192)
+        rows = torch.unique(torch.linspace(lo, hi - 1, 24).long())
         codes = q1.codes()[e]                                        # [N, K] on the GPU
         wd = (codes.float() * q1.scale[e].unsqueeze(-1)).t().cpu()   # [K, N]
-        ref = xd[ind[lo:hi] // k] @ wd
-        assert_parity(h[lo:hi], ref, torch.bfloat16, f"fp8 gate/up GEMM, expert {e}", tol=1e-2)
+        ref = xd[ind[rows] // k] @ wd
+        assert_parity(h[rows.cuda()], ref, torch.bfloat16, f"fp8 gate/up GEMM, expert {e}", tol=1e-2)
 
 
 @pytest.mark.parametrize("tiled", [True, False])

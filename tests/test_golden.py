@@ -59,8 +59,8 @@ def test_hip_layer_vector():
     out.backward(f["dout"].cuda())
     for got, key in ((out, "out"), (x.grad, "dx"), (w1.grad, "dw1"), (w2.grad, "dw2"),
                      (sc.grad, "dscores")):
-        assert moe_ref.rel_fro(got, f[key]) <= 2e-5, key
-        assert moe_ref.rel_max(got, f[key]) <= 2e-5, key
+        assert moe_ref.rel_fro(got, f[key]) <= 1e-5, key
+        assert moe_ref.rel_max(got, f[key]) <= 1e-5, key
 
 
 @pytest.mark.gpu

@@ -108,20 +108,28 @@ def test_package_op_level_loop_matches_the_oracle(gather, scatter, act):
     torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-5)
 
 
-def test_interleaved_copy_of_separate_gate_up_weights_is_cached_on_cpu():
+def test_separate_gate_up_weights_are_never_served_stale_on_cpu():
+    """Whatever route an update takes (in place, through .data, which leaves the version
+    counter alone, or a new storage), the next call interleaves the values of that moment."""
     from moe_explore.functional import topk_moe as layer
     from moe_explore.params import GLUParams
     g = seeded(6)
     gate, up, down = (torch.randn(s, generator=g) for s in ((3, 8, 6), (3, 8, 6), (3, 6, 8)))
     ep = GLUParams(gate, up, down, "swiglu")
     w_a = layer.expert_weights(ep)[0]
-    assert layer.expert_weights(ep)[0] is w_a
     assert torch.equal(w_a[..., 0::2], gate) and torch.equal(w_a[..., 1::2], up)
-    up.add_(1.0)                                      # written: the copy is rebuilt
+    up.add_(1.0)
+    assert torch.equal(layer.expert_weights(ep)[0][..., 1::2], up)
+    version = gate._version
+    gate.data.mul_(2.0)
+    up.data.copy_(torch.randn(3, 8, 6, generator=g))
+    assert gate._version == version
     w_b = layer.expert_weights(ep)[0]
-    assert w_b is not w_a and torch.equal(w_b[..., 1::2], up)
+    assert torch.equal(w_b[..., 0::2], gate) and torch.equal(w_b[..., 1::2], up)
     gate.requires_grad_(True)
+    gate.data.add_(1.0)
     w_c = layer.expert_weights(ep)[0]
+    assert torch.equal(w_c.detach()[..., 0::2], gate.detach())
     w_c.sum().backward()
     assert torch.equal(gate.grad, torch.ones_like(gate))
     assert layer.to_interleaved(ep).interleaved_weight.shape == (3, 8, 12)

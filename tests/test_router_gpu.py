@@ -93,6 +93,34 @@ def test_topk_router_matches_oracle(shape, dtype, softmax_first, normalize):
     assert so.shape == s.shape and io.shape == i.shape
 
 
+@pytest.mark.parametrize("E,topk", [(16, 4), (64, 8), (160, 6)])
+def test_masked_logits_are_chosen_last_and_never_twice(E, topk):
+    """Top-k before the softmax over tokens with fewer than k finite logits (a feature that
+    overflows to -inf for most experts): the finite experts are chosen, the rest of the k are
+    distinct experts with logit -inf and score 0 -- in every form of the selection (keys in
+    registers up to 16 experts a lane, in LDS beyond)."""
+    from moe_explore.params import TopkRouterParams
+    from moe_explore.router import topk_router, _fused_supported
+    T, d = 96, 64
+    x, w = _inputs(T, d, E, torch.bfloat16, seed=E)
+    finite = [3, E - 2]
+    x[:, 0] = 1e38                       # times -100, summed in fp32: -inf
+    w[0, :] = -100.0
+    w[0, finite] = 0.0
+    x, w = x.cuda(), w.cuda()
+    assert _fused_supported(x, w, topk, False)
+    s, i = topk_router(x, TopkRouterParams(w, topk, False, False))
+    s, i = s.float().cpu(), i.cpu()
+    assert (torch.sort(i, -1).values.diff(dim=-1) > 0).all(), "an expert chosen twice"
+    assert (i >= 0).all() and (i < E).all()
+    chosen = torch.zeros((T, E), dtype=torch.bool).scatter_(1, i, True)
+    assert chosen[:, finite].all(), "a finite logit was passed over for a masked one"
+    is_finite = torch.zeros(E, dtype=torch.bool)
+    is_finite[finite] = True
+    assert (s[~is_finite[i]] == 0).all()
+    torch.testing.assert_close(s.sum(-1), torch.ones(T), rtol=2e-2, atol=2e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", MANY_EXPERTS)
 @pytest.mark.parametrize("softmax_first,normalize", [(True, True), (False, False)])
@@ -120,14 +148,17 @@ def test_ernie_router_and_backward_with_384_experts():
     sg, ig = topk_router(xg, TopkRouterParams(wg, topk, True, True))
     g = torch.randn(sg.shape, generator=seeded(6))
     sg.backward(g.cuda())
-    xr = x.float().clone().requires_grad_(True)
-    wr = w.clone().requires_grad_(True)
-    pr = torch.softmax(xr @ wr, -1)
+    # fp32 router: 1e-5 against autograd in fp64 (logits rounded to fp32 as the kernel's are)
+    xr = x.double().requires_grad_(True)
+    wr = w.double().requires_grad_(True)
+    logits = xr @ wr
+    logits = logits + (logits.float().double() - logits).detach()
+    pr = torch.softmax(logits, -1)
     sr = torch.gather(pr, 1, ig.cpu())
     sr = sr / sr.sum(-1, keepdim=True)
-    sr.backward(g)
-    assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 1e-4
-    assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= 1e-4
+    sr.backward(g.double())
+    assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 1e-5
+    assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= 1e-5
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -183,13 +214,15 @@ def test_router_backward_matches_autograd(mode, dtype):
     s, i = router(xg, params)
     s.backward(g.cuda())
     idx = i.cpu()
-    # oracle: fp32 autograd through the same formulas with the same selection
-    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
+    # oracle: autograd through the same formulas with the same selection, in fp64 for the
+    # fp32 router (held to 1e-5) and in fp32 for the 16-bit one
+    cd = torch.float64 if dtype == torch.float32 else torch.float32
+    xr, wr = x.to(cd).requires_grad_(True), w.to(cd).requires_grad_(True)
     logits = xr @ wr
     if mode != "ernie":
         # the reference's matmul returns the logits in the dtype of x (router.py:22); rounding
         # has no gradient of its own (straight through)
-        logits = logits + (logits.to(dtype).float() - logits).detach()
+        logits = logits + (logits.to(dtype).to(cd) - logits).detach()
     if mode == "topk_first":
         sr = torch.softmax(torch.gather(logits, 1, idx), -1)
     else:
@@ -198,8 +231,8 @@ def test_router_backward_matches_autograd(mode, dtype):
             sr = sr / sr.sum(-1, keepdim=True)
         elif mode == "ernie":
             sr = sr / sr.sum(-1, keepdim=True).clamp_min(1e-12)
-    sr.backward(g.float())
-    tol = 1e-4 if dtype == torch.float32 else 2e-2   # the bar for bf16 results
+    sr.backward(g.to(cd))
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
     assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= tol
     assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= tol
 
@@ -247,10 +280,13 @@ def test_router_weight_gradient_with_many_tokens():
     assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 2e-2
 
 
-def test_ernie_router_gradients_with_many_tokens():
-    """fp32 router weight under bf16 activations, 8192 tokens and more: the backward products run
-    on 16-bit operands (dx) and over token groups on the K-grouped kernel (dW, returned in
-    fp32); against fp32 autograd with the same selection, at the bf16 bar."""
+@pytest.mark.parametrize("in_16_bits", [False, True])
+def test_ernie_router_gradients_with_many_tokens(in_16_bits):
+    """fp32 router weight under bf16 activations, 8192 tokens and more.  By default the weight
+    gradient comes from fp32 products (1e-5 against autograd in fp64 with the same selection;
+    dx leaves in bf16, at the bf16 bar); on request the backward products run on 16-bit
+    operands (dW over token groups on the K-grouped kernel, returned in fp32), at the bf16 bar."""
+    from moe_explore import router as router_module
     from moe_explore.params import ErnieRouterParams
     from moe_explore.router import ernie_router
     T, d, E, topk = 8192 + 33, 256, 64, 6
@@ -258,12 +294,18 @@ def test_ernie_router_gradients_with_many_tokens():
     bias = torch.randn(E, generator=seeded(9)) * 0.05
     g = torch.randn((T, topk), generator=seeded(10)).to(torch.bfloat16)
     xg, wg = x.cuda().requires_grad_(True), w.cuda().requires_grad_(True)
-    s, i = ernie_router(xg, ErnieRouterParams(wg, bias.cuda(), topk))
-    s.backward(g.cuda())
+    router_module.fp32_router_backward_in_16_bits(in_16_bits)
+    try:
+        s, i = ernie_router(xg, ErnieRouterParams(wg, bias.cuda(), topk))
+        s.backward(g.cuda())
+    finally:
+        router_module.fp32_router_backward_in_16_bits(False)
     assert wg.grad.dtype == torch.float32 and xg.grad.dtype == torch.bfloat16
-    xr, wr = x.float().requires_grad_(True), w.float().requires_grad_(True)
-    sr = torch.gather(torch.softmax(xr @ wr, -1), 1, i.cpu())
+    xr, wr = x.double().requires_grad_(True), w.double().requires_grad_(True)
+    logits = xr @ wr
+    logits = logits + (logits.float().double() - logits).detach()   # the kernel's fp32 logits
+    sr = torch.gather(torch.softmax(logits, -1), 1, i.cpu())
     sr = sr / sr.sum(-1, keepdim=True).clamp_min(1e-12)
-    sr.backward(g.float())
-    assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= 2e-2
+    sr.backward(g.double())
+    assert moe_ref.rel_fro(wg.grad.cpu(), wr.grad) <= (2e-2 if in_16_bits else 1e-5)
     assert moe_ref.rel_fro(xg.grad.cpu(), xr.grad) <= 2e-2

@@ -81,3 +81,37 @@ def test_noalloc_routing_python_wrapper_and_size_limit():
         big = torch.zeros(R, dtype=torch.int64, device="cuda")
         get_token_indices_into(big, E_big, torch.empty(R, dtype=torch.int64, device="cuda"),
                                torch.empty(E_big + 1, dtype=torch.int32, device="cuda"))
+
+
+def test_noalloc_routing_captured_into_a_graph_and_replayed():
+    """The call recorded into a HIP graph (after one eager call, which looks up the resident
+    buffer) and replayed twice in sequence on one stream with new expert ids each time, with
+    eager work of the same entry point between the replays: every replay equals the workspace
+    entry point on the ids of that moment."""
+    from moe_explore.expert_permute import get_token_indices, get_token_indices_into
+    g = torch.Generator().manual_seed(11)
+    T, k, E = 2000, 4, 32
+    ids = torch.randint(0, E, (T, k), generator=g).cuda()
+    ind = torch.empty(T * k, dtype=torch.int64, device="cuda")
+    gi = torch.empty(E + 1, dtype=torch.int32, device="cuda")
+    get_token_indices_into(ids, E, ind, gi)              # eager: resolves the buffer's address
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        get_token_indices_into(ids, E, ind, gi)
+    small = torch.randint(0, 5, (300,), generator=g).cuda()
+    for step in range(3):
+        ids.copy_(torch.randint(0, E, (T, k), generator=g))
+        ind.fill_(-1)
+        gi.fill_(-1)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = get_token_indices(ids, k, E, zero_prefix=True)
+        assert torch.equal(ind, want.indices) and torch.equal(gi, want.group_indices), f"replay {step}"
+        # eager use of the same buffer between the replays (other sizes: other counts in it)
+        e_ind = torch.empty(300, dtype=torch.int64, device="cuda")
+        e_gi = torch.empty(6, dtype=torch.int32, device="cuda")
+        get_token_indices_into(small, 5, e_ind, e_gi)
+        torch.cuda.synchronize()
+        e_want = get_token_indices(small, 1, 5, zero_prefix=True)
+        assert torch.equal(e_ind, e_want.indices) and torch.equal(e_gi, e_want.group_indices)
