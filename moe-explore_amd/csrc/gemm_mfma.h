@@ -82,17 +82,27 @@ struct Sched {
   // value is ~40 instructions): by GM * GN, nblk_n, GM and NT / ksplit
   int real_nt;  // NT / ksplit
   FastDiv by_block, by_nblk_n, by_gm, by_real_nt;
+  int band;       // > 0: bands of that many row blocks stay inside one expert (see make_sched)
+  int even_tail;  // the last two row blocks of a group share their rows evenly (see find_tile)
 };
 
 // The grid is a static bound: cdiv(P, BM) + E row blocks times the column tiles,
 // padded so that the GM x GN blocks tile it and their count is a multiple of 8.
-inline Sched make_sched(const MGemmArgs& g, int BM, int tpw = 1) {
+// band > 0: a band of `band` row blocks never crosses from one expert into the next (an expert
+// of n row blocks has cdiv(n, band) bands, the last one padded with empty slots), so that the
+// band x GN tiles an XCD works on at a time share GN weight panels instead of up to 2 GN; the
+// bound on the bands is then cdiv(cdiv(P, BM), band) + E.
+inline Sched make_sched(const MGemmArgs& g, int BM, int tpw = 1, int band = 0) {
   Sched s;
   s.tpw = tpw;
   s.ksplit = g.ksplit < 1 ? 1 : g.ksplit;
   s.NT = (static_cast<int>((g.N + BN - 1) / BN) + tpw - 1) / tpw * s.ksplit;
-  const int MT = static_cast<int>((g.P + BM - 1) / BM) + g.E;
-  s.GM = MT < 4 ? MT : 4;
+  int MT = static_cast<int>((g.P + BM - 1) / BM) + g.E;
+  if (band > 0) MT = band * (static_cast<int>(((g.P + BM - 1) / BM + band - 1) / band) + g.E);
+  s.band = band;
+  s.even_tail = 0;
+  const int gm = band > 0 ? band : 4;
+  s.GM = MT < gm ? MT : gm;
   s.GN = s.NT < 8 ? s.NT : 8;
   const int nblk_m = (MT + s.GM - 1) / s.GM;
   s.nblk_n = (s.NT + s.GN - 1) / s.GN;
@@ -170,11 +180,17 @@ __device__ __forceinline__ void leave_queues(unsigned* queue) {
 // (BM / 2 + ceil(r / 2) rounded up to 16, and the rest).  A block of few rows costs a workgroup
 // most of what a full one does (it streams the same weight panel; the matrix cores idle), while
 // two blocks of little more than BM / 2 rows each skip the multiplies of their dead 16-row
-// blocks: the pair takes about 1.3 instead of 1.6 full blocks' time.
-template <int BM, bool EVEN_TAIL = false>
+// blocks and take about as long as each other and as a full block, which keeps the work items
+// of a launch with few, long items alike.
+// BAND > 0: `mt` counts slots of expert-aligned bands of BAND row blocks (make_sched with
+// band): slot mt is row block (mt / BAND - bands before the expert) * BAND + mt % BAND of its
+// expert, or nothing when the expert has fewer row blocks.
+template <int BM>
 __device__ __forceinline__ void find_tile(const int32_t* __restrict__ gi, int E, int P, int mt,
-                                          int* sh) {
+                                          int* sh, bool EVEN_TAIL = false, int BAND = 0) {
   const int lane = threadIdx.x;
+  const int band = BAND > 0 ? mt / BAND : 0;
+  const int in_band = BAND > 0 ? mt - band * BAND : 0;
   int run = 0;
   bool done = false;
   for (int base = 0; base < E && !done; base += 64) {
@@ -187,16 +203,20 @@ __device__ __forceinline__ void find_tile(const int32_t* __restrict__ gi, int E,
       hi = hi > P ? P : hi;
     }
     const int tiles = hi > lo ? (hi - lo + BM - 1) / BM : 0;
-    int incl = tiles;
+    // what the scan counts: row blocks, or bands of them
+    const int units = BAND > 0 ? (tiles + BAND - 1) / BAND : tiles;
+    int incl = units;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
       int v = __shfl_up(incl, off, 64);
       if (lane >= off) incl += v;
     }
-    const int excl = run + incl - tiles;
-    const bool mine = mt >= excl && mt < excl + tiles;
+    const int excl = run + incl - units;
+    const int at = BAND > 0 ? band : mt;
+    const bool here = at >= excl && at < excl + units;
+    const int b = BAND > 0 ? (band - excl) * BAND + in_band : mt - excl;
+    const bool mine = here && b < tiles;
     if (mine) {
-      const int b = mt - excl;
       int first = lo + b * BM, last = hi;
       if (EVEN_TAIL && tiles >= 2 && b >= tiles - 2) {
         const int r = hi - lo - (tiles - 1) * BM;  // rows of the last block: 1 .. BM
@@ -210,7 +230,8 @@ __device__ __forceinline__ void find_tile(const int32_t* __restrict__ gi, int E,
       sh[1] = first;
       sh[2] = last;
     }
-    done = __ballot(mine) != 0;
+    done = __ballot(here) != 0;
+    if (done && __ballot(mine) == 0 && lane == 0) sh[0] = -1;  // a padding slot of the expert's last band
     run += __shfl(incl, 63, 64);
   }
   if (!done && lane == 0) sh[0] = -1;

@@ -469,3 +469,71 @@ def test_split_k_with_transposed_weights():
     summed = scale_and_reduce(parts, None, T, topk, N, nsplit=2)
     want = ref.view(T, topk, N).sum(1)
     assert_parity(summed, want, torch.bfloat16, "scale_and_reduce over parts and top-k")
+
+
+def _group_indices_of(sizes):
+    return torch.tensor([0] + list(torch.tensor(sizes).cumsum(0)), dtype=torch.int32)
+
+
+# rows per expert that exercise every case of the two tile orders: no rows, one short block, a
+# last block of 1, 128, 129 and 256 rows behind full ones, exactly four and eight blocks, five
+# and nine (a band of four and a remainder)
+TILE_ORDER_SIZES = [
+    [1036, 0, 5, 1024, 257, 384, 385, 2048, 2049, 1280, 1, 512],
+    [300, 260, 130, 0, 0, 769, 1152, 255, 256, 513],
+]
+
+
+@pytest.mark.parametrize("sizes", TILE_ORDER_SIZES)
+@pytest.mark.parametrize("transposed", [False, True])
+@pytest.mark.parametrize("activation", [None, "swiglu"])
+def test_expert_aligned_bands_with_long_k(sizes, transposed, activation):
+    """K = 4096 without split K: bands of four row blocks that stay inside one expert (padding
+    slots in an expert's last band are skipped).  Every expert on its own against the oracle."""
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    g = seeded(sum(sizes) + transposed)
+    R, E, K, N = sum(sizes), len(sizes), 4096, 512
+    x = randn((R, K), g, torch.bfloat16)
+    w = randn((E, K, N), g, torch.bfloat16, 1.0 / math.sqrt(K))
+    gi = _group_indices_of(sizes)
+    wc = w.cuda() if not transposed else w.transpose(1, 2).contiguous().cuda()
+    out = m_grouped_gemm(x.cuda(), _params(wc, gi.cuda(), None, False, False, R, 1, activation=activation),
+                         transpose_weight=transposed)
+    ref = moe_ref.grouped_matmul_gather_scatter(x, w, gi, activation_name=activation)
+    assert_parity(out, ref, torch.bfloat16, "bands, all rows")
+    for e, n in enumerate(sizes):
+        if n:
+            lo = int(gi[e])
+            assert_parity(out[lo:lo + n], ref[lo:lo + n], torch.bfloat16, f"expert {e} ({n} rows)")
+            last = lo + (n - 1) // 256 * 256     # the expert's last row block on its own
+            assert_parity(out[last:lo + n], ref[last:lo + n], torch.bfloat16, f"last block of expert {e}")
+
+
+@pytest.mark.parametrize("sizes", TILE_ORDER_SIZES)
+@pytest.mark.parametrize("transposed", [False, True])
+def test_even_last_row_blocks_with_split_k(sizes, transposed):
+    """Split K: a group whose last row block would hold at most 128 rows cuts its last two
+    blocks evenly instead; every row is still computed exactly once in each K part."""
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    g = seeded(sum(sizes) + 7 + transposed)
+    R, E, K, N = sum(sizes), len(sizes), 4096, 256
+    x = randn((R, K), g, torch.bfloat16)
+    w = randn((E, K, N), g, torch.bfloat16, 1.0 / math.sqrt(K))
+    gi = _group_indices_of(sizes)
+    perm = torch.randperm(R, generator=g)
+    wc = w.cuda() if not transposed else w.transpose(1, 2).contiguous().cuda()
+    p = _params(wc, gi.cuda(), perm.cuda(), False, True, R, 1)
+    parts = m_grouped_gemm(x.cuda(), p, transpose_weight=transposed, ksplit=2)
+    assert parts.shape == (2 * R, N), "the split was declined"
+    ref = moe_ref.grouped_matmul_gather_scatter(x, w, gi, perm, scatter=True, num_tokens=R, topk=1)
+    halves = [moe_ref.grouped_matmul_gather_scatter(x[:, h * 2048:(h + 1) * 2048], w[:, h * 2048:(h + 1) * 2048],
+                                                    gi, perm, scatter=True, num_tokens=R, topk=1)
+              for h in (0, 1)]
+    assert_parity(parts[:R], halves[0], torch.bfloat16, "first K part")
+    assert_parity(parts[R:], halves[1], torch.bfloat16, "second K part")
+    total = parts[:R].float() + parts[R:].float()
+    assert_parity(total, ref, torch.bfloat16, "sum of the K parts")
+    for e, n in enumerate(sizes):
+        if n:
+            rows = perm[int(gi[e]):int(gi[e]) + n]
+            assert_parity(total[rows.cuda()], ref[rows], torch.bfloat16, f"expert {e} ({n} rows)")
