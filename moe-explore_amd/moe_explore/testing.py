@@ -12,28 +12,21 @@ from moe_explore.params import MLPParams, GLUParams, TopkRouterParams, ErnieRout
 
 def torch_grouped_matmul_gather_scatter(a, params):
     """Per-expert matmul with optional gather, scatter, activation and combine
-    (``testing.py:9-50``)."""
-    dtype = a.dtype
-    b = params.weight
-    group_indices = params.group_indices
-    gather_indices = params.permute_indices // params.topk if params.gather else None
-    scatter_indices = params.permute_indices if params.scatter else None
-    c_rows = a.size(0) * params.topk if params.gather else a.size(0)
-    c = torch.zeros(c_rows, b.size(-1), device=a.device, dtype=dtype)
-    bounds = group_indices.tolist()
-    for i in range(b.size(0)):
-        glo, ghi = bounds[i], bounds[i + 1]
-        rows = a[gather_indices[glo:ghi]] if params.gather else a[glo:ghi]
-        prod = rows @ b[i]
-        if params.scatter:
-            c[scatter_indices[glo:ghi]] = prod
-        else:
-            c[glo:ghi] = prod
+    (``testing.py:9-50``).  All positions are gathered at once, every expert multiplies its
+    slice of them, and the products are scattered at once."""
+    weight, bounds = params.weight, params.group_indices.tolist()
+    rows = a.index_select(0, params.permute_indices // params.topk) if params.gather else a
+    products = [rows[lo:hi] @ weight[e] for e, (lo, hi) in enumerate(zip(bounds[:-1], bounds[1:]))]
+    c = torch.cat(products) if products else rows.new_zeros((0, weight.size(-1)))
+    if c.size(0) < rows.size(0):   # positions past the last group stay zero
+        c = torch.cat([c, c.new_zeros((rows.size(0) - c.size(0), c.size(1)))])
+    if params.scatter:
+        c = torch.zeros_like(c).index_copy_(0, params.permute_indices.to(torch.int64), c)
     if params.activation is not None:
         c = activation(c, params.activation)
     if params.scatter and params.scales is not None:
-        c = (c.view(params.num_tokens, params.topk, -1) * params.scales[..., None]).sum(1)
-    return c.to(dtype)
+        c = torch.einsum("tkn,tk->tn", c.view(params.num_tokens, params.topk, -1), params.scales.to(c.dtype))
+    return c.to(a.dtype)
 
 
 def torch_grouped_glu(a, params):
@@ -73,12 +66,10 @@ def random_routing(num_tokens, num_experts, topk, device, dtype):
 
 def random_skewed_routing(num_tokens, num_experts, topk, num_skewed_experts, skew_factor, device, dtype):
     """``num_skewed_experts`` experts are ``skew_factor`` times likelier (``testing.py:108-132``)."""
-    skewed = torch.randperm(num_experts)[:num_skewed_experts]
-    weights = torch.ones((num_tokens, num_experts), device=device, dtype=torch.float32)
-    weights[:, skewed] *= skew_factor
-    topk_indices = torch.multinomial(weights, num_samples=topk, replacement=False)
-    topk_scores, _ = random_routing(num_tokens, num_experts, topk, device, dtype)
-    return topk_scores, topk_indices
+    odds = torch.ones(num_experts, dtype=torch.float32)
+    odds[torch.randperm(num_experts)[:num_skewed_experts]] = skew_factor
+    topk_indices = torch.multinomial(odds.to(device).expand(num_tokens, num_experts), topk)
+    return random_routing(num_tokens, num_experts, topk, device, dtype)[0], topk_indices
 
 
 # Share (in percent, top-8) of tokens that reach each of OLMoE-1B-7B's 64 experts in the layer
@@ -118,14 +109,9 @@ def random_zipf_routing(num_tokens, num_experts, topk, device, dtype, s=1.2, gen
 
 def random_groups(num_tokens, num_groups, device):
     """``[0, r1 < r2 < ..., num_tokens]`` with random inner boundaries (``testing.py:212-224``)."""
-    indices = torch.arange(1, num_tokens - 1, device=device)
-    perm = torch.randperm(num_tokens - 2, device=device)
-    inner, _ = torch.sort(indices[perm[:num_groups - 1]])
-    group_indices = torch.empty(num_groups + 1, device=device, dtype=torch.int32)
-    group_indices[0] = 0
-    group_indices[1:-1] = inner
-    group_indices[-1] = num_tokens
-    return group_indices
+    inner = torch.randperm(num_tokens - 2, device=device)[:num_groups - 1] + 1   # distinct, in 1 .. n-2
+    ends = torch.tensor([0, num_tokens], device=device)
+    return torch.cat([ends[:1], torch.sort(inner).values, ends[1:]]).to(torch.int32)
 
 
 def uniform_weight_init(size, device, dtype):
@@ -191,18 +177,15 @@ def random_ernie_router(num_experts, hidden_dim, topk, device, dtype, dist=unifo
     )
 
 
+# one unit in the last place of 1.0 per dtype, as the reference's tolerance rule takes it
+_EPS = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 1e-6}
+
+
 def assert_close(a, b):
-    """Tolerance rule of the reference's tests (``testing.py:340-357``)."""
-    if a.dtype is torch.bfloat16:
-        eps = 0.0078125
-    elif a.dtype is torch.float16:
-        eps = 0.0009765625
-    elif a.dtype is torch.float32:
-        eps = 1e-6
-    else:
+    """Tolerance rule of the reference's tests (``testing.py:340-357``): absolute tolerance
+    ``min(1e-2, k * max * eps / 100)``, relative ``sqrt(k) * eps / 10`` for rows of ``k`` values."""
+    if a.dtype not in _EPS:
         raise ValueError(f"Invalid dtype: {a.dtype}")
-    k = a.size(-1)
-    m = max(a.max(), b.max()).item()
-    atol = min(1e-2, k * m * eps * 1e-2)
-    rtol = math.sqrt(k) * eps * 1e-1
-    torch.testing.assert_close(a, b, atol=atol, rtol=rtol)
+    eps, k = _EPS[a.dtype], a.size(-1)
+    largest = max(a.max(), b.max()).item()
+    torch.testing.assert_close(a, b, atol=min(1e-2, k * largest * eps * 1e-2), rtol=math.sqrt(k) * eps * 1e-1)
