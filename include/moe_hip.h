@@ -102,14 +102,15 @@ MOE_API int moe_route_preprocess(const void* expert_ids, int idx_bytes, int64_t 
  * bit.  The per-chunk counts live in a buffer of moe_route_noalloc_max_bytes() bytes (4 MiB)
  * that is part of the library image on every device: calls with
  * moe_route_workspace_bytes(R, E) above that (ceil(R / 512) * E > 2^20) return
- * MOE_ERR_WORKSPACE.  All calls on one device share that buffer: calls that may overlap in
- * time (different streams) race; calls on one stream are ordered and safe.  Nothing in the
- * buffer has to be cleared between calls.  Under graph capture the captured launches keep
- * using that one buffer: replays of a graph that holds this call must not overlap each other
- * or an eager call on the same device (replays launched into one stream are ordered and
- * safe).  The first call on a device looks up the buffer's address and is refused with
- * MOE_ERR_HIP while its stream is being captured: make one call (R = 0 will do) before the
- * capture begins.
+ * MOE_ERR_WORKSPACE.  All calls on one device share that buffer, and nothing in it has to be
+ * cleared between calls.  Eager calls cannot race on it: calls on one stream are ordered, and a
+ * call on another stream than the call before makes its stream wait (hipStreamWaitEvent) for that
+ * call's launches, so calls from several streams run one after the other.  Under graph capture
+ * nothing is waited for or recorded and the captured launches keep using that one buffer:
+ * replays of a graph that holds this call must not overlap each other or an eager call on the
+ * same device (replays launched into one stream are ordered and safe).  The first call on a
+ * device looks up the buffer's address and creates the event; it is refused with MOE_ERR_HIP
+ * while its stream is being captured: make one call (R = 0 will do) before the capture begins.
  */
 MOE_API size_t moe_route_noalloc_max_bytes(void);
 MOE_API int moe_route_preprocess_noalloc(const void* expert_ids, int idx_bytes, int64_t R, int E,

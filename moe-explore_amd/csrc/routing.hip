@@ -215,28 +215,43 @@ int check_route_args(const void* expert_ids, int idx_bytes, int64_t R, int E,
 constexpr size_t kScratchWords = size_t(1) << 20;  // 4 MiB
 static __device__ __align__(256) int32_t scratch[kScratchWords];
 
-// `stream`: the stream of the call that asks.  The first call on a device looks the address up
-// (which may load the code object); that is not done while `stream` is being captured into a
-// graph: such a call is refused, and the caller makes one call outside the capture first.
-int32_t* scratch_of_current_device(hipStream_t stream) {
-  constexpr int kMaxDevices = 64;
-  static int32_t* of_device[kMaxDevices];
-  static std::mutex lock;
+// One record per device: the buffer's address, and who used it last.  Eager calls from different
+// streams would race on the buffer, so a call on another stream than the one before first makes
+// its stream wait for an event recorded behind that call's launches: calls then run one after the
+// other whatever streams they come from.  (Under graph capture nothing is recorded or waited for:
+// the graph's replays are ordered by whoever launches them, see the header.)
+struct ScratchOfDevice {
+  int32_t* ptr = nullptr;
+  hipEvent_t done = nullptr;     // behind the launches of the last eager call
+  hipStream_t last = nullptr;    // the stream of that call
+  bool used = false;
+};
+constexpr int kMaxScratchDevices = 64;
+ScratchOfDevice g_scratch_of[kMaxScratchDevices];
+std::mutex g_scratch_lock;
+
+// The buffer of the current device for a call on `stream`, or nullptr (error set).  The first call
+// on a device looks the address up (which may load the code object) and creates the event; that is
+// not done while `stream` is being captured into a graph: such a call is refused, and the caller
+// makes one call outside the capture first.  *capturing tells whether `stream` is being captured.
+int32_t* acquire_scratch(hipStream_t stream, ScratchOfDevice** rec, bool* capturing) {
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
-  if (err != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+  if (err != hipSuccess || dev < 0 || dev >= kMaxScratchDevices) {
     fail(MOE_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(err));
     return nullptr;
   }
-  std::lock_guard<std::mutex> hold(lock);
-  if (of_device[dev] == nullptr) {
-    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-    err = hipStreamIsCapturing(stream, &capture);
-    if (err != hipSuccess) {
-      fail(MOE_ERR_HIP, "hipStreamIsCapturing: %s", hipGetErrorString(err));
-      return nullptr;
-    }
-    if (capture != hipStreamCaptureStatusNone) {
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  err = hipStreamIsCapturing(stream, &capture);
+  if (err != hipSuccess) {
+    fail(MOE_ERR_HIP, "hipStreamIsCapturing: %s", hipGetErrorString(err));
+    return nullptr;
+  }
+  *capturing = capture != hipStreamCaptureStatusNone;
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  ScratchOfDevice& d = g_scratch_of[dev];
+  if (d.ptr == nullptr) {
+    if (*capturing) {
       fail(MOE_ERR_HIP, "the first moe_route_preprocess_noalloc call on a device looks up its "
                         "resident buffer and cannot run under stream capture: make one call "
                         "(any size, R = 0 will do) before the capture begins");
@@ -248,9 +263,32 @@ int32_t* scratch_of_current_device(hipStream_t stream) {
       fail(MOE_ERR_HIP, "hipGetSymbolAddress(routing scratch): %s", hipGetErrorString(err));
       return nullptr;
     }
-    of_device[dev] = static_cast<int32_t*>(p);
+    err = hipEventCreateWithFlags(&d.done, hipEventDisableTiming);
+    if (err != hipSuccess) {
+      fail(MOE_ERR_HIP, "hipEventCreateWithFlags: %s", hipGetErrorString(err));
+      return nullptr;
+    }
+    d.ptr = static_cast<int32_t*>(p);
   }
-  return of_device[dev];
+  if (!*capturing && d.used && d.last != stream) {
+    err = hipStreamWaitEvent(stream, d.done, 0);
+    if (err != hipSuccess) {
+      fail(MOE_ERR_HIP, "hipStreamWaitEvent: %s", hipGetErrorString(err));
+      return nullptr;
+    }
+  }
+  *rec = &d;
+  return d.ptr;
+}
+
+// Behind the launches of an eager call.
+int release_scratch(ScratchOfDevice* rec, hipStream_t stream) {
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  const hipError_t err = hipEventRecord(rec->done, stream);
+  if (err != hipSuccess) return fail(MOE_ERR_HIP, "hipEventRecord: %s", hipGetErrorString(err));
+  rec->last = stream;
+  rec->used = true;
+  return MOE_OK;
 }
 
 }  // namespace
@@ -285,8 +323,13 @@ extern "C" int moe_route_preprocess_noalloc(const void* expert_ids, int idx_byte
                 "routing of %lld slots over %d experts needs %zu bytes of scratch; the resident "
                 "buffer of moe_route_preprocess_noalloc has %zu (use moe_route_preprocess with a "
                 "workspace)", (long long)R, E, need, kScratchWords * sizeof(int32_t));
-  int32_t* const counts = scratch_of_current_device(static_cast<hipStream_t>(stream_));
+  hipStream_t stream = static_cast<hipStream_t>(stream_);
+  ScratchOfDevice* rec = nullptr;
+  bool capturing = false;
+  int32_t* const counts = acquire_scratch(stream, &rec, &capturing);
   if (counts == nullptr) return MOE_ERR_HIP;
-  return route_preprocess_launch(expert_ids, idx_bytes, R, E, indices_out, group_indices_out,
-                                 inclusive_out, counts, static_cast<hipStream_t>(stream_));
+  const int rc = route_preprocess_launch(expert_ids, idx_bytes, R, E, indices_out, group_indices_out,
+                                         inclusive_out, counts, stream);
+  if (rc != MOE_OK || capturing) return rc;
+  return release_scratch(rec, stream);
 }

@@ -537,3 +537,31 @@ def test_even_last_row_blocks_with_split_k(sizes, transposed):
         if n:
             rows = perm[int(gi[e]):int(gi[e]) + n]
             assert_parity(total[rows.cuda()], ref[rows], torch.bfloat16, f"expert {e} ({n} rows)")
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+@pytest.mark.parametrize("ksplit", [1, 2])
+def test_tile_orders_with_many_random_groups(seed, ksplit):
+    """More experts than one pass of the tile lookup scans (64), random group sizes from 0 to a
+    few row blocks, K = 4096: expert-aligned bands (ksplit 1) and the even last pair of row
+    blocks (ksplit 2) must visit every row block exactly once."""
+    from moe_explore.triton_kernels.m_grouped_gemm import m_grouped_gemm
+    g = seeded(100 + seed)
+    E, K, N = 150, 4096, 256
+    sizes = torch.randint(0, 700, (E,), generator=g)
+    sizes[torch.randint(0, E, (20,), generator=g)] = 0
+    sizes[torch.randint(0, E, (5,), generator=g)] = torch.tensor([256, 512, 1024, 1, 1300])
+    sizes = sizes.tolist()
+    R = sum(sizes)
+    x = randn((R, K), g, torch.bfloat16)
+    w = randn((E, K, N), g, torch.bfloat16, 1.0 / math.sqrt(K))
+    gi = _group_indices_of(sizes)
+    out = m_grouped_gemm(x.cuda(), _params(w.cuda(), gi.cuda(), None, False, False, R, 1), ksplit=ksplit)
+    if ksplit == 2:
+        assert out.shape == (2 * R, N)
+        out = out[:R].float() + out[R:].float()
+    ref = moe_ref.grouped_matmul_gather_scatter(x, w, gi)
+    assert_parity(out, ref, torch.bfloat16, "all rows")
+    # row by row: a row block visited twice or not at all shows as a row that is off
+    err = (out.float().cpu() - ref).norm(dim=1) / ref.norm(dim=1).clamp_min(1e-6)
+    assert err.max().item() <= 2e-2, f"row {int(err.argmax())} is off by {err.max().item():.3e}"

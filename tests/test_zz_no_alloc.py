@@ -115,3 +115,25 @@ def test_noalloc_routing_captured_into_a_graph_and_replayed():
         torch.cuda.synchronize()
         e_want = get_token_indices(small, 1, 5, zero_prefix=True)
         assert torch.equal(e_ind, e_want.indices) and torch.equal(e_gi, e_want.group_indices)
+
+
+def test_noalloc_routing_from_two_streams_back_to_back():
+    """Calls issued on two streams without any synchronisation between them share the one
+    resident buffer; the entry point orders them itself (the second stream waits for the first
+    call's launches), so both results are right."""
+    from moe_explore.expert_permute import get_token_indices, get_token_indices_into
+    g = torch.Generator().manual_seed(23)
+    cases = [(98304, 64), (60000, 48), (98304, 64), (30000, 8)]
+    ids = [torch.randint(0, E, (R,), generator=g).cuda() for R, E in cases]
+    outs = [(torch.full((R,), -1, dtype=torch.int64, device="cuda"),
+             torch.full((E + 1,), -1, dtype=torch.int32, device="cuda")) for R, E in cases]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for i, ((R, E), x, (ind, gi)) in enumerate(zip(cases, ids, outs)):
+            with torch.cuda.stream(streams[i % 2]):
+                get_token_indices_into(x, E, ind, gi)
+    torch.cuda.synchronize()
+    for (R, E), x, (ind, gi) in zip(cases, ids, outs):
+        want = get_token_indices(x, 1, E, zero_prefix=True)
+        assert torch.equal(ind, want.indices) and torch.equal(gi, want.group_indices)
