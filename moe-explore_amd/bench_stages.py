@@ -22,6 +22,9 @@ each prints its own short table, and the kernel trace / counters of the profiler
              weight-streaming rate and TFLOP/s
   gemms      the six grouped GEMMs of a Mixtral-shape training step one by one (median of event
              pairs), with the bench's routing and with evenly loaded experts
+  combine    the down projection of the Mixtral-shape layer with its top-k combine, two ways: rows
+             stored in slot order (split K) + scale_and_reduce, as the layer runs it, and the
+             weighted scatter-add fused into the GEMM's store (fp32 atomics, m_grouped_gemm(combine=True))
   digest     the digest of the dominant kernel's sources that a profile summary records
 """
 import argparse
@@ -37,7 +40,7 @@ for p in (ROOT, HERE):
 
 import bench  # noqa: E402  (the headline benchmark: config, inputs, digest)
 
-STAGES = ["kernel", "copy", "router", "passes", "configs23", "models", "fp32", "fp8", "gemms", "digest"]
+STAGES = ["kernel", "copy", "router", "passes", "configs23", "models", "fp32", "fp8", "gemms", "combine", "digest"]
 
 
 def main():
@@ -294,6 +297,42 @@ def main():
                 m_grouped_gemm(x, gp, out=a_out)
         torch.cuda.synchronize()
         print("launched the gate/up grouped GEMM x %d" % args.steps)
+        return
+    if args.stage == "combine":
+        from moe_explore.functional.scale_and_reduce import scale_and_reduce
+        from moe_explore.functional.topk_moe import _ksplit_for
+
+        def median_ms(fn):
+            for _ in range(args.warmup):
+                fn()
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                   for _ in range(args.steps)]
+            for s, e in evs:
+                s.record()
+                fn()
+                e.record()
+            torch.cuda.synchronize()
+            return sorted(s.elapsed_time(e) for s, e in evs)[len(evs) // 2]
+
+        with torch.no_grad():
+            p = get_token_indices(idx, k, E, zero_prefix=True)
+            a = torch.randn((R, ff), device=dev, dtype=torch.bfloat16)
+            dn = MGroupedGEMMParams(w2, p.group_indices, p.indices, False, True, T, k, scales=scores)
+            ks = _ksplit_for(R, E, d, ff)
+
+            def two_passes():
+                y = m_grouped_gemm(a, dn, ksplit=ks)
+                return scale_and_reduce(y, scores, T, k, d, nsplit=y.size(0) // R)
+
+            t_gemm = median_ms(lambda: m_grouped_gemm(a, dn, ksplit=ks))
+            t_two = median_ms(two_passes)
+            t_fused = median_ms(lambda: m_grouped_gemm(a, dn, combine=True))
+            ref, got = two_passes().float(), m_grouped_gemm(a, dn, combine=True).float()
+            err = ((got - ref).norm() / ref.norm()).item()
+        print("down projection + top-%d combine, T=%d d=%d ff=%d E=%d (%.0f M output elements scattered):" % (k, T, d, ff, E, R * d / 1e6))
+        print("  GEMM storing rows in slot order (split K = %d)        %7.3f ms" % (ks, t_gemm))
+        print("  ... + scale_and_reduce (the layer's path)            %7.3f ms" % t_two)
+        print("  GEMM with the weighted scatter-add fused (fp32 atomics) %7.3f ms   (rel. difference of the results %.1e)" % (t_fused, err))
         return
     if args.stage == "gemms":
         from moe_explore.functional.topk_moe import _ksplit_for
