@@ -22,6 +22,8 @@ each prints its own short table, and the kernel trace / counters of the profiler
              weight-streaming rate and TFLOP/s
   gemms      the six grouped GEMMs of a Mixtral-shape training step one by one (median of event
              pairs), with the bench's routing and with evenly loaded experts
+  routings   the four M-grouped GEMMs of a Mixtral-shape training step with other routings: five
+             more seeds of router logits at 4096 tokens, then 3000, 6144, 8192 and 2048 tokens
   combine    the down projection of the Mixtral-shape layer with its top-k combine, two ways: rows
              stored in slot order (split K) + scale_and_reduce, as the layer runs it, and the
              weighted scatter-add fused into the GEMM's store (fp32 atomics, m_grouped_gemm(combine=True))
@@ -40,7 +42,7 @@ for p in (ROOT, HERE):
 
 import bench  # noqa: E402  (the headline benchmark: config, inputs, digest)
 
-STAGES = ["kernel", "copy", "router", "passes", "configs23", "models", "fp32", "fp8", "gemms", "combine", "digest"]
+STAGES = ["kernel", "copy", "router", "passes", "configs23", "models", "fp32", "fp8", "gemms", "routings", "combine", "digest"]
 
 
 def main():
@@ -333,6 +335,52 @@ def main():
         print("  GEMM storing rows in slot order (split K = %d)        %7.3f ms" % (ks, t_gemm))
         print("  ... + scale_and_reduce (the layer's path)            %7.3f ms" % t_two)
         print("  GEMM with the weighted scatter-add fused (fp32 atomics) %7.3f ms   (rel. difference of the results %.1e)" % (t_fused, err))
+        return
+    if args.stage == "routings":
+        from moe_explore.functional.topk_moe import _ksplit_for
+        from moe_explore.hip_kernels.m_grouped_gemm import m_grouped_gemm_glu_bwd
+        from moe_explore.router import route_from_logits
+
+        def timed(fn):
+            for _ in range(args.warmup):
+                fn()
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                   for _ in range(args.steps)]
+            for s, e in evs:
+                s.record()
+                fn()
+                e.record()
+            torch.cuda.synchronize()
+            return sorted(s.elapsed_time(e) for s, e in evs)[len(evs) // 2]
+
+        del x, dout
+        total = 0.0
+        for tokens, seed in ((T, 1), (T, 2), (T, 3), (T, 4), (T, 5), (3000, 6), (6144, 7), (8192, 8), (2048, 9)):
+            g = torch.Generator(device=dev).manual_seed(seed)
+            xs = torch.randn(tokens, d, device=dev, generator=g).to(torch.bfloat16)
+            ds = torch.randn(tokens, d, device=dev, generator=g).to(torch.bfloat16)
+            sc, ii = route_from_logits(torch.randn(tokens, E, device=dev, generator=g), k, True, True,
+                                       torch.bfloat16)
+            with torch.no_grad():
+                p = get_token_indices(ii, k, E, zero_prefix=True)
+                gi, ind = p.group_indices, p.indices
+                gu = MGroupedGEMMParams(w1, gi, ind, True, False, tokens, k, activation="swiglu")
+                a, h = m_grouped_gemm(xs, gu, save_preact=True)
+                dn = MGroupedGEMMParams(w2, gi, ind, False, True, tokens, k, scales=sc)
+                pf = MGroupedGEMMParams(w2, gi, ind, True, False, tokens, k, scales=sc)
+                dh, _, _ = m_grouped_gemm_glu_bwd(ds, pf, h, "swiglu", transpose_weight=True, want_dscale=True)
+                px = MGroupedGEMMParams(w1, gi, ind, False, True, tokens, k)
+                ks, ksx = _ksplit_for(tokens * k, E, d, ff), _ksplit_for(tokens * k, E, d, 2 * ff)
+                ms = [timed(lambda: m_grouped_gemm(xs, gu, save_preact=True)),
+                      timed(lambda: m_grouped_gemm(a, dn, ksplit=ks)),
+                      timed(lambda: m_grouped_gemm_glu_bwd(ds, pf, h, "swiglu", transpose_weight=True,
+                                                           want_dscale=True)),
+                      timed(lambda: m_grouped_gemm(dh, px, transpose_weight=True, ksplit=ksx))]
+            total += sum(ms)
+            print("T=%d seed %d rows %s split K %d/%d: gate/up %.3f  down %.3f  G fused %.3f  dX %.3f  sum %.3f ms" % (
+                tokens, seed, (gi[1:] - gi[:-1]).tolist(), ks, ksx, *ms, sum(ms)), flush=True)
+            del xs, ds, a, h, dh
+        print("total %.3f ms" % total)
         return
     if args.stage == "gemms":
         from moe_explore.functional.topk_moe import _ksplit_for
