@@ -234,6 +234,8 @@ std::mutex g_scratch_lock;
 // on a device looks the address up (which may load the code object) and creates the event; that is
 // not done while `stream` is being captured into a graph: such a call is refused, and the caller
 // makes one call outside the capture first.  *capturing tells whether `stream` is being captured.
+// The caller holds g_scratch_lock from here until release_scratch has returned, so that two host
+// threads cannot both pass the wait for the call before them and then launch side by side.
 int32_t* acquire_scratch(hipStream_t stream, ScratchOfDevice** rec, bool* capturing) {
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);
@@ -248,7 +250,6 @@ int32_t* acquire_scratch(hipStream_t stream, ScratchOfDevice** rec, bool* captur
     return nullptr;
   }
   *capturing = capture != hipStreamCaptureStatusNone;
-  std::lock_guard<std::mutex> hold(g_scratch_lock);
   ScratchOfDevice& d = g_scratch_of[dev];
   if (d.ptr == nullptr) {
     if (*capturing) {
@@ -283,7 +284,6 @@ int32_t* acquire_scratch(hipStream_t stream, ScratchOfDevice** rec, bool* captur
 
 // Behind the launches of an eager call.
 int release_scratch(ScratchOfDevice* rec, hipStream_t stream) {
-  std::lock_guard<std::mutex> hold(g_scratch_lock);
   const hipError_t err = hipEventRecord(rec->done, stream);
   if (err != hipSuccess) return fail(MOE_ERR_HIP, "hipEventRecord: %s", hipGetErrorString(err));
   rec->last = stream;
@@ -326,6 +326,7 @@ extern "C" int moe_route_preprocess_noalloc(const void* expert_ids, int idx_byte
   hipStream_t stream = static_cast<hipStream_t>(stream_);
   ScratchOfDevice* rec = nullptr;
   bool capturing = false;
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
   int32_t* const counts = acquire_scratch(stream, &rec, &capturing);
   if (counts == nullptr) return MOE_ERR_HIP;
   const int rc = route_preprocess_launch(expert_ids, idx_bytes, R, E, indices_out, group_indices_out,
